@@ -151,7 +151,7 @@ typedef float hy_v16f __attribute__((ext_vector_type(16)));
 // Epilogues: STORE = the float32 products; GLU = gate / up pairs -> activation in the matrix type; ACTMUL = gelu_tanh(product) times an
 // entry of a per-token table row (mul_table[mul_rows[m]][mul_col0 + feature]) in the matrix type (the per-layer token input).
 enum { HY_EPI_STORE = 0, HY_EPI_GLU = 1, HY_EPI_ACTMUL = 2 };
-struct HyGlu { float limit, alpha, shift; const void* mul_table; const int* mul_rows; int mul_ld, mul_col0; };
+struct HyGlu { float limit, alpha, shift; const void* mul_table; const int* mul_rows; int mul_ld, mul_col0; int act; };      // act 1: gelu_tanh(g) u
 __device__ __forceinline__ float hy_gelu_tanh(float z) { return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z))); }
 template <typename T>
 __device__ __forceinline__ float hy_actmul(float a, int m, int feature, const HyGlu& p) {
@@ -159,6 +159,7 @@ __device__ __forceinline__ float hy_actmul(float a, int m, int feature, const Hy
 }
 __device__ __forceinline__ float hy_glu(float g, float u, const HyGlu& p) {
     if (p.limit > 0.f) { g = fminf(g, p.limit); u = fminf(fmaxf(u, -p.limit), p.limit); }
+    if (p.act == 1) return hy_gelu_tanh(g) * u;
     return g * hy_sigmoid(p.alpha * g) * (u + p.shift);
 }
 
@@ -305,7 +306,7 @@ static __global__ __launch_bounds__(256) void hy_gemm_kernel(const T* __restrict
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int m = m0 + wm * (BM / 2) + i * 32 + 8 * (r >> 2) + rbase + (r & 3);
-                    if (m < M && f < ld_act) hy_st(act + (size_t)m * ld_act + f, hy_glu(acc[i][j][r], acc[i][j + 1][r], glu));
+                    if (m < M && f < ld_act && 2 * f < N) hy_st(act + (size_t)m * ld_act + f, hy_glu(acc[i][j][r], acc[i][j + 1][r], glu));
                 }
             }
     }
@@ -422,55 +423,101 @@ static __global__ __launch_bounds__(256) void hy_matvec_kernel(const T* __restri
 // One wavefront per (token, head): query heads are normalised (unit root mean square, optional) and turned by their position (optional)
 // in place, key heads likewise on their way to the key rows of the slot, value heads are normalised (optional), turned (optional) and
 // written to the value rows.  proj row = [.. q (H x D) .. k (G x D) .. v (G x V) ..].
-// Rotary turn: entry i of the first `dims` pairs with entry i + dims / 2 and the pair (u, v) becomes (u cos a - v sin a, v cos a + u sin a),
-// a = pos * freq[i] in float32; freq is a table the host made (base^(-2 i / dims), divided for q / k by the position scaling).
+// Rotary turn: entry i of the first `dims` pairs with entry i + dims / 2 (interleaved: entry 2 i with entry 2 i + 1) and the pair (u, v)
+// becomes (u cos a - v sin a, v cos a + u sin a), a = pos * freq[i] in float32; freq is a table the host made (base^(-2 i / dims),
+// divided for q / k by the position scaling).  An entry is (src + bias) * r * weight before it turns (bias, weight: null = absent).
 struct HyRot {
     int qk_dims; const float* qk_freq;       // q / k: first qk_dims entries turn; 0 = none
     int v_norm;                              // values: unit root mean square per head
     const float* v_freq;                     // values: all V entries turn (null = none)
+    int interleaved;                         // q / k pairs are (2 i, 2 i + 1)
 };
-__device__ __forceinline__ void hy_turn_store(float* __restrict__ dst, const float* __restrict__ src, int D, int dims, const float* __restrict__ freq, float pos, float r, int lane) {
+// further inputs of the cache writers (null = absent): a bias per projection row, added first; weights of the norm over a whole
+// projection (unit_norm = 2)
+struct HyPrepX { const float* bias; const float* qn; const float* kn; const float* rowr; };
+__device__ __forceinline__ void hy_turn_store(float* __restrict__ dst, const float* __restrict__ src, int D, int dims, const float* __restrict__ freq, float pos, float r, int lane,
+                                              int interleaved = 0, const float* __restrict__ bias = nullptr, const float* __restrict__ w = nullptr) {
     const int half = dims >> 1;
+    auto val = [&](int d) { return (src[d] + (bias ? bias[d] : 0.f)) * r * (w ? w[d] : 1.f); };
     for (int d = lane; d < half; d += 64) {
         float sn, cs;
         sincosf(pos * freq[d], &sn, &cs);
-        const float u = src[d] * r, v = src[d + half] * r;
-        dst[d] = u * cs - v * sn;
-        dst[d + half] = v * cs + u * sn;
+        const int i0 = interleaved ? 2 * d : d, i1 = interleaved ? 2 * d + 1 : d + half;
+        const float u = val(i0), v = val(i1);
+        dst[i0] = u * cs - v * sn;
+        dst[i1] = v * cs + u * sn;
     }
-    for (int d = dims + lane; d < D; d += 64) dst[d] = src[d] * r;
+    for (int d = dims + lane; d < D; d += 64) dst[d] = val(d);
 }
 static __global__ __launch_bounds__(64) void hy_attn_prep_kernel(float* __restrict__ proj, int ld, int q_off, int k_off, int v_off, int H, int G, int D, int V,
                                                                  int unit_norm, float eps, float* __restrict__ kc, float* __restrict__ vc, size_t slot_stride,
-                                                                 const int* __restrict__ dyn, HyRot rot) {
+                                                                 const int* __restrict__ dyn, HyRot rot, HyPrepX x = HyPrepX{}) {
     const int t = blockIdx.x, hh = blockIdx.y, lane = threadIdx.x;
     const int pos = dyn[0] + t;
     const size_t slot = (size_t)dyn[1] * slot_stride;
     if (hh < H + G) {
         const bool isq = hh < H;
-        float* src = proj + (size_t)t * ld + (isq ? q_off + hh * D : k_off + (hh - H) * D);
+        const int col = isq ? q_off + hh * D : k_off + (hh - H) * D;
+        float* src = proj + (size_t)t * ld + col;
+        const float* bias = x.bias ? x.bias + col : nullptr;
+        const float* w = nullptr;
         float r = 1.f;
-        if (unit_norm) {
+        if (unit_norm == 2) {          // over the whole projection: hy_rowrms_kernel has left 1 / rms of the token's q and k rows
+            r = x.rowr[2 * t + (isq ? 0 : 1)];
+            w = (isq ? x.qn : x.kn) + (isq ? hh : hh - H) * D;
+        } else if (unit_norm) {
             float ss = 0.f;
-            for (int d = lane; d < D; d += 64) ss += src[d] * src[d];
+            for (int d = lane; d < D; d += 64) { const float v = src[d] + (bias ? bias[d] : 0.f); ss += v * v; }
             ss = hy_wave_sum(ss);
             r = 1.f / sqrtf(ss / (float)D + eps);
         }
         float* dst = isq ? src : kc + slot + (size_t)pos * (G * D) + (hh - H) * D;
-        if (isq && !unit_norm && !rot.qk_dims) return;
-        hy_turn_store(dst, src, D, rot.qk_dims, rot.qk_freq, (float)pos, r, lane);      // a lane reads both entries of its pairs before it writes them
+        if (isq && !unit_norm && !rot.qk_dims && !bias) return;
+        hy_turn_store(dst, src, D, rot.qk_dims, rot.qk_freq, (float)pos, r, lane, rot.interleaved, bias, w);      // a lane reads both entries of its pairs before it writes them
     } else {
         const int g = hh - H - G;
         const float* src = proj + (size_t)t * ld + v_off + g * V;
+        const float* bias = x.bias ? x.bias + v_off + g * V : nullptr;
         float* dst = vc + slot + (size_t)pos * (G * V) + g * V;
         float r = 1.f;
         if (rot.v_norm) {
             float ss = 0.f;
-            for (int d = lane; d < V; d += 64) ss += src[d] * src[d];
+            for (int d = lane; d < V; d += 64) { const float v = src[d] + (bias ? bias[d] : 0.f); ss += v * v; }
             ss = hy_wave_sum(ss);
             r = 1.f / sqrtf(ss / (float)V + eps);
         }
-        hy_turn_store(dst, src, V, rot.v_freq ? V : 0, rot.v_freq, (float)pos, r, lane);
+        hy_turn_store(dst, src, V, rot.v_freq ? V : 0, rot.v_freq, (float)pos, r, lane, 0, bias);
+    }
+}
+
+// 1 / sqrt(mean((x + bias)^2) + eps) over two column ranges of every token's projection row (the whole q projection and the whole k
+// projection): out[2 t], out[2 t + 1].  Runs before the cache writers rewrite q in place.
+static __global__ __launch_bounds__(256) void hy_rowrms_kernel(const float* __restrict__ proj, int ld, int off0, int len0, int off1, int len1,
+                                                               const float* __restrict__ bias, float eps, float* __restrict__ out) {
+    __shared__ float red[4];
+    const int t = blockIdx.x, which = blockIdx.y, off = which ? off1 : off0, len = which ? len1 : len0;
+    const float* row = proj + (size_t)t * ld + off;
+    float ss = 0.f;
+    for (int d = threadIdx.x; d < len; d += 256) { const float v = row[d] + (bias ? bias[off + d] : 0.f); ss += v * v; }
+    ss = hy_block_sum<256>(ss, red);
+    if (threadIdx.x == 0) out[2 * t + which] = 1.f / sqrtf(ss / (float)len + eps);
+}
+
+// Pooled rows of a cache: block b holds positions b P .. b P + P - 1 and its pooled key / value is the mean of the block's cached rows
+// (summed in position order).  One workgroup per block that the step completes (its last position lies in the step) and cache
+// (blockIdx.y = 0 keys, 1 values).
+static __global__ __launch_bounds__(256) void hy_pool_kernel(const float* __restrict__ kc, const float* __restrict__ vc, float* __restrict__ pk, float* __restrict__ pv,
+                                                             int ldk, int ldv, int P, size_t slot_stride, const int* __restrict__ dyn, int n) {
+    const int b = dyn[0] / P + blockIdx.x;
+    if ((b + 1) * P > dyn[0] + n) return;
+    const size_t slot = (size_t)dyn[1] * slot_stride;
+    const int ld = blockIdx.y ? ldv : ldk;
+    const float* src = (blockIdx.y ? vc : kc) + slot + (size_t)b * P * ld;
+    float* dst = (blockIdx.y ? pv : pk) + slot + (size_t)b * ld;
+    for (int c = threadIdx.x; c < ld; c += 256) {
+        float a = 0.f;
+        for (int j = 0; j < P; ++j) a += src[(size_t)j * ld + c];
+        dst[c] = a / (float)P;
     }
 }
 
@@ -553,6 +600,9 @@ struct HyAttnArgs {
     int kt;                             // keys per tile: 64, or 32 / 16 / 8 where 64 rows do not fit LDS (lanes >= kt idle in the score phase)
     int shared_kv;                      // keys and values are the same rows (latent attention): staged once
     int window, keep;                   // query at position i sees key j <= i if i - j < window or j < keep; window <= 0: every earlier key
+    // pool > 0 (with a window): pooled rows pk / pv (laid out like kc / vc, one row per block of `pool` positions); query i also sees
+    // the pooled rows of blocks b with b pool + pool - 1 <= i - window
+    const float* pk; const float* pv; int pool;
 };
 constexpr int HY_KT = 64;
 
@@ -633,15 +683,27 @@ static __global__ __launch_bounds__(256) void hy_attn_kernel(HyAttnArgs a) {
     const int win = a.window > 0 ? a.window : 0x3fffffff;
     const int minpos = pos0 + (rb * 4 * RW) / hpg;
     const int lo_t = max(0, minpos - win + 1) / KT, hi_t = maxpos / KT;
-    const int nk = min((a.keep + KT - 1) / KT, lo_t), nv = nk + hi_t - lo_t + 1;
+    const int nk = min((a.keep + KT - 1) / KT, lo_t);
     const int pos_lo = pos0 + min(rows - 1, row0) / hpg;   // the wavefront's earliest row
+    // pooled blocks a position sees: those that end at or before pos - window; the tiles of pooled rows come first in the list
+    const int P = a.pool;
+    int nbr[RW];
+#pragma unroll
+    for (int r = 0; r < RW; ++r) nbr[r] = P > 0 ? max(0, pr[r] - win + 1) / P : 0;
+    const int nb_wg = P > 0 ? max(0, maxpos - win + 1) / P : 0, nb_hi = P > 0 ? max(0, pos_hi - win + 1) / P : 0;
+    const int np_t = (nb_wg + KT - 1) / KT, nv = np_t + nk + hi_t - lo_t + 1;
+    const float* pkc = P > 0 ? a.pk + slot + (size_t)g * dk : kc;
+    const float* pvc = P > 0 ? a.pv + slot + (size_t)g * dv : vc;
     for (int vt = split; vt < nv; vt += a.nsplit) {
-        const int j0 = (vt < nk ? vt : lo_t + vt - nk) * KT;
+        const bool pooled = vt < np_t;
+        const int wt = vt - np_t;
+        const int j0 = (pooled ? vt : wt < nk ? wt : lo_t + wt - nk) * KT;
         __syncthreads();                                   // previous tile fully consumed (and sQ written, first time)
-        hy_stage_rows(sK, ks, kc, ldk, dk, j0, KT, maxpos, veck);
-        if (!a.shared_kv) hy_stage_rows(sV, dv, vc, ldv, dv, j0, KT, maxpos, vecv);
+        hy_stage_rows(sK, ks, pooled ? pkc : kc, ldk, dk, j0, KT, pooled ? nb_wg - 1 : maxpos, veck);
+        if (!a.shared_kv) hy_stage_rows(sV, dv, pooled ? pvc : vc, ldv, dv, j0, KT, pooled ? nb_wg - 1 : maxpos, vecv);
         __syncthreads();
-        if (j0 > pos_hi || (j0 >= a.keep && j0 + KT <= pos_lo - win + 1)) continue;      // uniform per wavefront: no row of it sees a key of this tile
+        // uniform per wavefront: no row of it sees a key of this tile
+        if (pooled ? j0 >= nb_hi : (j0 > pos_hi || (j0 >= a.keep && j0 + KT <= pos_lo - win + 1))) continue;
         float s[RW];
 #pragma unroll
         for (int r = 0; r < RW; ++r) s[r] = 0.f;
@@ -670,7 +732,8 @@ static __global__ __launch_bounds__(256) void hy_attn_kernel(HyAttnArgs a) {
         const int j = j0 + lane;
 #pragma unroll
         for (int r = 0; r < RW; ++r) {
-            s[r] = (j <= pr[r] && lane < KT && (pr[r] - j < win || j < a.keep)) ? s[r] - slope[r] * (float)(pr[r] - j) : -INFINITY;
+            if (pooled) s[r] = (j < nbr[r] && lane < KT) ? s[r] : -INFINITY;
+            else s[r] = (j <= pr[r] && lane < KT && (pr[r] - j < win || j < a.keep)) ? s[r] - slope[r] * (float)(pr[r] - j) : -INFINITY;
             const float mn = fmaxf(m[r], hy_wave_max(s[r]));
             const bool any = mn > -INFINITY;                         // false: this row has seen no key yet (its keys start in a later tile of the split)
             const float corr = any ? expf(m[r] - mn) : 1.f;          // exp(-inf) = 0 the first time
@@ -682,7 +745,7 @@ static __global__ __launch_bounds__(256) void hy_attn_kernel(HyAttnArgs a) {
             if (lane < KT) myP[lane * RW + r] = p;
         }
         __builtin_amdgcn_wave_barrier();
-        const int jn = min(KT, pos_hi - j0 + 1);
+        const int jn = min(KT, (pooled ? nb_hi : pos_hi + 1) - j0);
         int jj = 0;
         for (; jj + 4 <= jn; jj += 4) {                     // four keys at a time, reads first
             float pj[4][RW], vv[4][DVL];
@@ -727,18 +790,21 @@ static __global__ __launch_bounds__(256) void hy_attn_kernel(HyAttnArgs a) {
     }
 }
 
-// out[t][h dv + c] = gate * sum_s e^(m_s - M) acc_s[c] / (sum_s e^(m_s - M) l_s + sink e^(-M)),  M = max(m_s, sink ? 0 : -inf).
+// out[t][h dv + c] = out_mul * gate * sum_s e^(m_s - M) acc_s[c] / (sum_s e^(m_s - M) l_s + sink e^(z - M)),  M = max(m_s, sink ? z : -inf),
+// z = sink_w ? sink_w[h] : 0 (a learned logit per head, or one plain unit).
 // gate_mode 1: gate[t][h dv + c], 2: gate[t][h] (one per head).  v_freq != null: the head's output is turned back by the token's
 // position over all dv entries (pairs c, c + dv / 2, angle -pos v_freq[c]) before the gate.
 template <typename TO>
 static __global__ __launch_bounds__(64) void hy_attn_merge_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml, int H, int dv, int nsplit,
                                                                   int sink, const float* __restrict__ gate, int ldg, int gate_mode, TO* __restrict__ out, int ldo,
-                                                                  const float* __restrict__ v_freq, const int* __restrict__ dyn) {
+                                                                  const float* __restrict__ v_freq, const int* __restrict__ dyn,
+                                                                  const float* __restrict__ sink_w = nullptr, float out_mul = 1.f) {
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     const size_t o = ((size_t)t * H + h) * nsplit;
-    float M = sink ? 0.f : -INFINITY;
+    const float z = sink_w ? sink_w[h] : 0.f;
+    float M = sink ? z : -INFINITY;
     for (int s = 0; s < nsplit; ++s) M = fmaxf(M, part_ml[2 * (o + s)]);
-    float den = sink ? expf(-M) : 0.f;
+    float den = sink ? expf(z - M) : 0.f;
     for (int s = 0; s < nsplit; ++s) {
         const float ms = part_ml[2 * (o + s)];
         if (ms > -INFINITY) den += expf(ms - M) * part_ml[2 * (o + s) + 1];
@@ -754,7 +820,7 @@ static __global__ __launch_bounds__(64) void hy_attn_merge_kernel(const float* _
     const float ghead = (gate && gate_mode == 2) ? hy_sigmoid(gate[(size_t)t * ldg + h]) : 1.f;
     auto put = [&](int c, float v) {
         if (gate && gate_mode != 2) v *= hy_sigmoid(gate[(size_t)t * ldg + h * dv + c]);
-        hy_st(out + (size_t)t * ldo + h * dv + c, v * ghead);
+        hy_st(out + (size_t)t * ldo + h * dv + c, v * ghead * out_mul);
     };
     if (v_freq) {
         const int half = dv >> 1;
@@ -802,55 +868,98 @@ static __global__ __launch_bounds__(256) void hy_conv_tail_kernel(const float* _
     }
 }
 
-// Recurrence S_t = e^(-e^(A_log) dt_t) S_(t-1) + dt_t B_t x_t^T,  y_t = S_t^T C_t + D x_t  per head, S = N x P, dt = softplus(raw + bias).
+// Recurrence S_t = a_t S_(t-1) + b_t k_t x_t^T,  y_t = S_t^T q_t + D x_t  per head, S = N x P (keys / queries of N entries, values of P).
+// Three sources of a_t, b_t (HyScanArgs.mode): 0, a state-space layer: dt = softplus(raw + bias), a = e^(-e^(A_log) dt), b = dt, keys
+// and queries shared by the heads of a group; 1, gates that a kernel before this one left per (token, head) (hy_mem_gates_kernel);
+// 2, a fixed decay per head, b = 1.  Keys and queries may turn by their position on the way into LDS (rot: first `dims` entries, pairs
+// (i, i + dims / 2) or (2 i, 2 i + 1), angle = position * freq[i]) and are multiplied by k_mul / q_mul afterwards.  ones_col: the last of
+// the P columns has x = 1 whatever the token (it then carries n_t = a n + b k, the normaliser of a matrix memory, and y's last column
+// is n_t . q_t).
 // Workgroup = one head x 4 wavefronts; a wavefront = 64 / NG value columns, a column's N states spread over NG lanes (lane i holds the NL
-// states n = i NL .. i NL + NL - 1, in registers for the whole portion; NG NL >= N).  Tokens run in order, TB at a time: the block's B and C
-// rows (padded to NG NL), its x columns, step sizes and decays are staged in LDS by all four wavefronts (coalesced); every wavefront then
-// walks the TB tokens reading its B / C slice with 16-byte LDS reads and leaves its lanes' partial sums of y in LDS; the sums over a
+// states n = i NL .. i NL + NL - 1, in registers for the whole portion; NG NL >= N).  Tokens run in order, TB at a time: the block's key and
+// query rows (padded to NG NL), its x columns, a and b are staged in LDS by all four wavefronts (coalesced); every wavefront then
+// walks the TB tokens reading its key / query slice with 16-byte LDS reads and leaves its lanes' partial sums of y in LDS; the sums over a
 // column's NG lanes, the skip term and the (coalesced) store of y follow once per block, off the recurrence's critical path.  The slot's
 // state is read at the start (zero at position 0) and written at the end.
+struct HyScanRot { int dims; const float* freq; int interleaved; };
+struct HyScanArgs {
+    const float* ksrc; int ldk, k_off, k_hstride;      // key of (t, head): ksrc + t ldk + k_off + (head / heads-per-group) k_hstride
+    const float* qsrc; int ldq, q_off, q_hstride;
+    const float* xsrc; int ldx, x_off;                 // x of (t, head, column): xsrc + t ldx + x_off + head Px + column, Px = P - ones_col
+    float k_mul, q_mul;
+    HyScanRot rot;
+    int mode;
+    const float* dtsrc; int ld_dt, dt_off; const float* dt_bias; const float* A_log; const float* Dp;      // mode 0 (Dp: null = no skip term)
+    const float* ga; const float* gb;                  // mode 1: [n][heads]
+    const float* decay;                                // mode 2: [heads]
+    int ones_col;
+    int heads, P, N, G, NG, TB;
+    float* state; size_t slot_stride; const int* dyn; int n;
+    float* y; int ldy;                                 // y of (t, head, column): y + t ldy + head P + column
+};
+__device__ __forceinline__ float hy_scan_fetch(const float* __restrict__ row, int nn, int N, const HyScanRot& rot, float pos) {
+    if (nn >= N) return 0.f;
+    if (nn >= rot.dims) return row[nn];
+    const int half = rot.dims >> 1;
+    const int i = rot.interleaved ? nn >> 1 : (nn < half ? nn : nn - half);
+    const bool first = rot.interleaved ? !(nn & 1) : nn < half;
+    const int other = rot.interleaved ? nn ^ 1 : (first ? nn + half : nn - half);
+    float sn, cs;
+    sincosf(pos * rot.freq[i], &sn, &cs);
+    return first ? row[nn] * cs - row[other] * sn : row[nn] * cs + row[other] * sn;
+}
 template <int NL>
-static __global__ __launch_bounds__(256) void hy_ssm_scan_kernel(const float* __restrict__ proj, int ld, int dt_off, const float* __restrict__ conv, int ch,
-                                                                 int heads, int P, int N, int G, int NG, int TB, const float* __restrict__ dt_bias,
-                                                                 const float* __restrict__ A_log, const float* __restrict__ Dp, float* __restrict__ state,
-                                                                 size_t slot_stride, const int* __restrict__ dyn, int n, float* __restrict__ y) {
+static __global__ __launch_bounds__(256) void hy_ssm_scan_kernel(HyScanArgs a) {
     extern __shared__ __attribute__((aligned(16))) float smem[];
+    const int P = a.P, N = a.N, NG = a.NG, TB = a.TB, n = a.n, Px = P - (a.ones_col ? 1 : 0);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, head = blockIdx.y, ng = lane % NG;
     const int cpw = 64 / NG, cols = 4 * cpw, col0 = blockIdx.x * cols, myc = wave * cpw + lane / NG, p = col0 + myc, Ns = NG * NL;
     const bool livep = p < P;
-    const int inner = heads * P, g = head / (heads / G);
-    const int b_off = inner + g * N, c_off = inner + G * N + g * N;
+    const int g = head / (a.heads / a.G);
+    const float* kbase = a.ksrc + a.k_off + (size_t)g * a.k_hstride;
+    const float* qbase = a.qsrc + a.q_off + (size_t)g * a.q_hstride;
+    const float* xbase = a.xsrc + a.x_off + (size_t)head * Px;
     float* sB = smem;                    // [TB][Ns]
     float* sC = sB + TB * Ns;            // [TB][Ns]
     float* sY = sC + TB * Ns;            // [TB][256] partial sums of y per lane
     float* sX = sY + TB * 256;           // [TB][cols]
-    float* sDt = sX + TB * cols;         // [TB] step size, [TB] decay
-    float* S = state + (size_t)dyn[1] * slot_stride + (size_t)head * N * P;
-    const bool fresh = dyn[0] == 0;
+    float* sDt = sX + TB * cols;         // [TB] b_t, [TB] a_t
+    float* S = a.state + (size_t)a.dyn[1] * a.slot_stride + (size_t)head * N * P;
+    const int pos0 = a.dyn[0];
+    const bool fresh = pos0 == 0;
     float s[NL];
 #pragma unroll
     for (int i = 0; i < NL; ++i) {
         const int nn = ng * NL + i;
         s[i] = (!fresh && livep && nn < N) ? S[(size_t)nn * P + p] : 0.f;
     }
-    const float na = -expf(A_log[head]), dtb = dt_bias[head], dd = Dp[head];
+    const float na = a.mode == 0 ? -expf(a.A_log[head]) : 0.f, dtb = a.mode == 0 ? a.dt_bias[head] : 0.f, dd = (a.mode == 0 && a.Dp) ? a.Dp[head] : 0.f;
+    const float fixed = a.mode == 2 ? a.decay[head] : 0.f;
     for (int t0 = 0; t0 < n; t0 += TB) {
         const int tb = min(TB, n - t0);
         __syncthreads();
         for (int i = tid; i < tb * Ns; i += 256) {
             const int t = i / Ns, nn = i - t * Ns;
-            const float* cr = conv + (size_t)(t0 + t) * ch;
-            sB[i] = nn < N ? cr[b_off + nn] : 0.f;
-            sC[i] = nn < N ? cr[c_off + nn] : 0.f;
+            const float pos = (float)(pos0 + t0 + t);
+            sB[i] = hy_scan_fetch(kbase + (size_t)(t0 + t) * a.ldk, nn, N, a.rot, pos) * a.k_mul;
+            sC[i] = hy_scan_fetch(qbase + (size_t)(t0 + t) * a.ldq, nn, N, a.rot, pos) * a.q_mul;
         }
         for (int i = tid; i < tb * cols; i += 256) {
             const int t = i / cols, c = i - t * cols;
-            sX[i] = col0 + c < P ? conv[(size_t)(t0 + t) * ch + head * P + col0 + c] : 0.f;
+            sX[i] = col0 + c < Px ? xbase[(size_t)(t0 + t) * a.ldx + col0 + c] : (col0 + c < P ? 1.f : 0.f);
         }
         if (tid < tb) {
-            const float dt = hy_softplus(proj[(size_t)(t0 + tid) * ld + dt_off + head] + dtb);
-            sDt[tid] = dt;
-            sDt[TB + tid] = expf(na * dt);
+            if (a.mode == 0) {
+                const float dt = hy_softplus(a.dtsrc[(size_t)(t0 + tid) * a.ld_dt + a.dt_off + head] + dtb);
+                sDt[tid] = dt;
+                sDt[TB + tid] = expf(na * dt);
+            } else if (a.mode == 1) {
+                sDt[tid] = a.gb[(size_t)(t0 + tid) * a.heads + head];
+                sDt[TB + tid] = a.ga[(size_t)(t0 + tid) * a.heads + head];
+            } else {
+                sDt[tid] = 1.f;
+                sDt[TB + tid] = fixed;
+            }
         }
         __syncthreads();
         for (int t = 0; t < tb; ++t) {
@@ -874,7 +983,7 @@ static __global__ __launch_bounds__(256) void hy_ssm_scan_kernel(const float* __
             if (col0 + c >= P) continue;
             float v = 0.f;
             for (int k = 0; k < NG; ++k) v += sY[t * 256 + c * NG + k];
-            y[(size_t)(t0 + t) * inner + head * P + col0 + c] = fmaf(dd, sX[i], v);
+            a.y[(size_t)(t0 + t) * a.ldy + head * P + col0 + c] = fmaf(dd, sX[i], v);
         }
     }
 #pragma unroll
@@ -884,10 +993,74 @@ static __global__ __launch_bounds__(256) void hy_ssm_scan_kernel(const float* __
     }
 }
 
+// Gates of a matrix memory with exponential gating, per (token, head), from the raw gate projections z_i, z_f (+ biases):
+//   i = cap tanh(z_i / cap), f = logsigmoid(cap tanh(z_f / cap)), m_t = max(f + m_(t-1), i) (m before the first token is 0),
+//   ga = e^(f + m_(t-1) - m_t), gb = e^(i - m_t), ge = e^(-m_t).
+// One workgroup per head: i and f of a block of tokens are made by all threads, one thread walks the chain of maxima (two operations a
+// token), all threads finish ga / gb / ge.  The slot keeps m.
+constexpr int HY_GATE_TB = 1024;
+static __global__ __launch_bounds__(256) void hy_mem_gates_kernel(const float* __restrict__ proj, int ld, int i_off, int f_off, const float* __restrict__ bias, float cap,
+                                                                  int heads, float* __restrict__ mstate, size_t slot_stride, const int* __restrict__ dyn, int n,
+                                                                  float* __restrict__ ga, float* __restrict__ gb, float* __restrict__ ge) {
+    __shared__ float si[HY_GATE_TB], sf[HY_GATE_TB], sm[HY_GATE_TB + 1];
+    const int head = blockIdx.x, tid = threadIdx.x;
+    float* mp = mstate + (size_t)dyn[1] * slot_stride + head;
+    float mprev = dyn[0] == 0 ? 0.f : *mp;
+    for (int t0 = 0; t0 < n; t0 += HY_GATE_TB) {
+        const int tb = min(HY_GATE_TB, n - t0);
+        __syncthreads();
+        for (int t = tid; t < tb; t += 256) {
+            const float* row = proj + (size_t)(t0 + t) * ld;
+            const float zi = row[i_off + head] + (bias ? bias[i_off + head] : 0.f), zf = row[f_off + head] + (bias ? bias[f_off + head] : 0.f);
+            si[t] = cap * tanhf(zi / cap);
+            const float fr = cap * tanhf(zf / cap);
+            sf[t] = fminf(fr, 0.f) - log1pf(expf(-fabsf(fr)));          // log sigmoid
+        }
+        __syncthreads();
+        if (tid == 0) {
+            float m = mprev;
+            sm[0] = m;
+            for (int t = 0; t < tb; ++t) { m = fmaxf(sf[t] + m, si[t]); sm[t + 1] = m; }
+        }
+        __syncthreads();
+        for (int t = tid; t < tb; t += 256) {
+            const size_t o = (size_t)(t0 + t) * heads + head;
+            ga[o] = expf(sf[t] + sm[t] - sm[t + 1]);
+            gb[o] = expf(si[t] - sm[t + 1]);
+            ge[o] = expf(-sm[t + 1]);
+        }
+        mprev = sm[tb];          // every thread reads the same value before the next block's barrier
+    }
+    if (tid == 0) *mp = mprev;
+}
+
+// What leaves a matrix memory: one wavefront per (token, head).  o = y[0 .. V) of the head (row stride ldy, P = V or V + 1 columns per
+// head), divided by max(|y[V]|, ge[t][head]) + 1e-6 where the memory has a normaliser (ge != null); then o / sqrt(mean(o^2) + eps), times
+// w[head V + c] (null = none), times act(gate[t][g_off + head V + c]) (act = silu, or sigmoid for gate_act 1), times out_mul, stored in the
+// matrix type at out[t ldo + head V + c].
+template <typename TO>
+static __global__ __launch_bounds__(64) void hy_mem_out_kernel(const float* __restrict__ y, int ldy, int P, int V, const float* __restrict__ ge, int heads,
+                                                               const float* __restrict__ w, const float* __restrict__ gate, int ldg, int g_off, int gate_act,
+                                                               float eps, float out_mul, TO* __restrict__ out, int ldo) {
+    const int t = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+    const float* row = y + (size_t)t * ldy + (size_t)head * P;
+    float inv = 1.f;
+    if (ge) inv = 1.f / (fmaxf(fabsf(row[V]), ge[(size_t)t * heads + head]) + 1e-6f);
+    float ss = 0.f;
+    for (int c = lane; c < V; c += 64) { const float v = row[c] * inv; ss += v * v; }
+    ss = hy_wave_sum(ss);
+    const float r = 1.f / sqrtf(ss / (float)V + eps);
+    for (int c = lane; c < V; c += 64) {
+        const float z = gate[(size_t)t * ldg + g_off + head * V + c];
+        const float gv = gate_act == 1 ? hy_sigmoid(z) : hy_silu(z);
+        hy_st(out + (size_t)t * ldo + head * V + c, row[c] * inv * r * (w ? w[head * V + c] : 1.f) * gv * out_mul);
+    }
+}
+
 // y * silu(z), unit root mean square per part (ngroups equal parts of inner), times the weight
 template <typename TO>
 static __global__ __launch_bounds__(256) void hy_gated_norm_kernel(const float* __restrict__ y, const float* __restrict__ proj, int ld, int z_off, int inner,
-                                                                   int ngroups, const float* __restrict__ w, float eps, TO* __restrict__ out) {
+                                                                   int ngroups, const float* __restrict__ w, float eps, TO* __restrict__ out, int ldo) {
     __shared__ float red[4];
     const int t = blockIdx.x, grp = blockIdx.y, len = inner / ngroups, c0 = grp * len;
     float ss = 0.f;
@@ -899,6 +1072,6 @@ static __global__ __launch_bounds__(256) void hy_gated_norm_kernel(const float* 
     const float r = 1.f / sqrtf(ss / (float)len + eps);
     for (int i = threadIdx.x; i < len; i += 256) {
         const float v = y[(size_t)t * inner + c0 + i] * hy_silu(proj[(size_t)t * ld + z_off + c0 + i]);
-        hy_st(out + (size_t)t * inner + c0 + i, v * r * w[c0 + i]);
+        hy_st(out + (size_t)t * ldo + c0 + i, v * r * w[c0 + i]);
     }
 }

@@ -7,7 +7,7 @@
 
 // ---- residual update ----------------------------------------------------------------------------------------------------------------
 // One workgroup per token.  In this order, every part optional (null pointer = absent):
-//   x += ga * sum_z ya[z]                       ya: a sublayer's output, possibly as K-split parts; ga = sigmoid(gate_z[t * gate_ld]) or 1
+//   x += ya_mul * ga * sum_z ya[z]              ya: a sublayer's output (or several sublayers' outputs), possibly as K-split parts; ga = sigmoid(gate_z[t * gate_ld]) or 1
 //   x += sum_k eo[pair_row[t top + k]]          the routed experts' down projections of this token
 //   x += yc / sqrt(mean(yc^2) + eps) * cw       a unit-RMS normed input with a plain weight
 //   hist_out[t] = x;  x = sum_j mix[j] hist[j][t], j < n_mix, where hist[n_mix - 1] is hist_out (what the layer leaves is an average over
@@ -16,7 +16,7 @@
 //   h = x / sqrt(mean(x^2) + eps) * norm_w in the matrix type (the next sublayer's input; norm_w already holds any offset)
 struct HyResid {
     float* x; int W;
-    const float* ya; int ya_parts; size_t ya_stride; const float* gate_z; int gate_ld;
+    const float* ya; int ya_parts; size_t ya_stride; const float* gate_z; int gate_ld; float ya_mul;
     const float* eo; const int* pair_row; int top;
     const float* yc; const float* cw;
     float* hist; size_t hist_stride; int n_mix; const float* mix;      // hist_out = hist + (n_mix - 1) hist_stride
@@ -59,7 +59,7 @@ static __global__ __launch_bounds__(NT) void hy_resid_kernel(HyResid a, TO* __re
         ss = hy_block_sum<NT>(ss, red);
         cr = 1.f / sqrtf(ss / (float)W + a.eps);
     }
-    const float ga = a.gate_z ? hy_sigmoid(a.gate_z[(size_t)t * a.gate_ld]) : 1.f;
+    const float ga = (a.gate_z ? hy_sigmoid(a.gate_z[(size_t)t * a.gate_ld]) : 1.f) * a.ya_mul;
     float ss = 0.f, keep[HY_RC][V];
     int it = 0;
     for (int w = threadIdx.x * V; w < W; w += NT * V, ++it) {

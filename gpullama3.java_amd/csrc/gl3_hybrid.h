@@ -6,6 +6,7 @@
 #include "gl3_ctx.h"
 
 constexpr int HY_KSPLIT = 4;     // most partial sums a K-split output / down projection leaves for the streams kernel to add
+constexpr int HY_YPARTS = 2 * HY_KSPLIT;      // copies of y: in a parallel block the mixer's and the feed-forward's parts lie side by side
 
 struct HyMat {                 // [rows][ld] of the plan's matrix type (bfloat16 or float32), K-contiguous, zero padded
     void* w = nullptr;
@@ -14,10 +15,21 @@ struct HyMat {                 // [rows][ld] of the plan's matrix type (bfloat16
 
 struct HyLayer {
     gl3_layer_desc d{};
-    // fused input projection of the mixer: attention q | k | v | gate; latent q | latent | gate; ssm z | x | B | C | dt
+    // fused input projection of the mixer: attention q | k | v | gate; latent q | latent | gate; ssm z | x | B | C | dt; matrix memory
+    // q | k | v | gate | input gate | forget gate.  A layer with two mixers side by side keeps the second one in `side`: its rows follow
+    // the first mixer's in the layer's proj, its output columns follow the first mixer's in mixo and in o (the offsets below count from
+    // the start of the fused row; proj, o and pbias of `side` are unused / borrowed)
     HyMat proj;
-    int q_off = 0, k_off = 0, v_off = 0, g_off = 0, c_off = 0;
-    HyMat o;                   // the mixer's output projection [width x heads * vdim]
+    int q_off = 0, k_off = 0, v_off = 0, g_off = 0, c_off = 0, i_off = 0, f_off = 0;
+    int o0 = 0;                // first column of this mixer's heads in mixo and o
+    int mo_total = 0;          // columns of o: this mixer's heads * vdim plus the side mixer's
+    float out_mul = 1.f;
+    HyLayer* side = nullptr;   // owned
+    HyMat o;                   // the mixer's output projection [width x mo_total]
+    float* pbias = nullptr;    // bias per row of the fused projection (null: no mixer of the layer has biases)
+    float *qn = nullptr, *kn = nullptr, *sink = nullptr;      // attention: weights of the whole-projection q / k norms, learned sink logits
+    float* decay = nullptr;    // matrix memory: fixed decay per head
+    size_t off_pk = 0, off_pv = 0, off_m = 0;                 // float offsets inside a slot: pooled key / value rows, running maxima of the gates
     HyMat gu, down;            // feed-forward (in a mixture of experts: the shared expert): gate / up rows in blocks of 32 + 32 (2 ff_pad rows), down [width x ff_pad]
     int ff_pad = 0;
     int dense_ff = 0;          // width of that feed-forward (d.ff, or d.shared_ff in a mixture of experts; 0 = none)
@@ -44,6 +56,8 @@ struct gl3_hybrid_state {
     bool f32 = false;          // GL3_FLAG_F32_COMPUTE
     int S = 1, W = 0, mb = 1, n_seqs = 1, want_cap = 1;
     bool plain = false;        // one residual stream without stream tables (gl3_model_desc.streams == 0)
+    bool parallel = false;     // plain: one norm per layer, mixer and feed-forward read it and are added together (gl3_model_desc.parallel_block)
+    float resid_mul = 1.f, logit_mul = 1.f;
     float emb_scale = 1.f, norm_offset = 0.f;
     int side_dim = 0, side_ld = 0, max_top = 0;
     bool depth = false;
@@ -63,6 +77,8 @@ struct gl3_hybrid_state {
     std::vector<int> len;      // tokens a slot holds
     // scratch of one portion of a step (<= mb tokens)
     float *X = nullptr, *proj = nullptr, *y = nullptr, *conv = nullptr, *ssm_y = nullptr, *qa = nullptr, *oc = nullptr, *kx = nullptr, *vx = nullptr, *part_acc = nullptr, *part_ml = nullptr;
+    float *gates = nullptr, *rowr = nullptr;     // matrix memory: a, b, e^(-m) per (token, head), [3][mb][max heads]; attention: 1 / rms of the whole q and k rows [mb][2]
+    int max_heads = 1;
     void *h = nullptr, *mixo = nullptr, *xw = nullptr;
     float *logits = nullptr, *taps = nullptr, *ones = nullptr;
     int *tokens = nullptr, *dyn = nullptr, *want = nullptr;

@@ -53,15 +53,18 @@ static int32_t hy_alloc_mat(gl3_ctx* ctx, HyMat& m, int rows, int k, int ld) {
 }
 
 // ---- shapes -----------------------------------------------------------------------------------------------------------------------
-static int hy_gate_rows(const gl3_layer_desc& d) { return d.out_gate == 2 ? d.heads : d.out_gate ? d.heads * d.vdim : 0; }
+static int hy_gate_rows(const gl3_layer_desc& d) { return d.mixer == GL3_MIX_MEMORY ? d.heads * d.vdim : d.out_gate == 2 ? d.heads : d.out_gate ? d.heads * d.vdim : 0; }
+// rows of ONE mixer's part of the fused input projection
 static int hy_proj_rows(const gl3_layer_desc& d) {
     switch (d.mixer) {
         case GL3_MIX_ATTENTION: return d.heads * d.dim + d.kv_heads * d.dim + d.kv_heads * d.vdim + hy_gate_rows(d);
         case GL3_MIX_LATENT: return d.heads * d.dim + d.kv_rank + hy_gate_rows(d);
+        case GL3_MIX_MEMORY: return 2 * d.heads * d.dim + 2 * d.heads * d.vdim + (d.mem_gates == GL3_MEM_EXP_GATES ? 2 * d.heads : 0);
         default: return 2 * d.heads * d.vdim + 2 * d.groups * d.state + d.heads;
     }
 }
 static int hy_mix_out(const gl3_layer_desc& d) { return d.heads * d.vdim; }
+static bool hy_has_bias(const gl3_layer_desc& d) { return (d.mixer == GL3_MIX_ATTENTION && d.qk_bias) || (d.mixer == GL3_MIX_MEMORY && d.mem_gates == GL3_MEM_EXP_GATES); }
 static int hy_conv_ch(const gl3_layer_desc& d) { return d.heads * d.vdim + 2 * d.groups * d.state; }
 
 static const char* hy_check_layer(const gl3_layer_desc& d) {
@@ -75,8 +78,10 @@ static const char* hy_check_layer(const gl3_layer_desc& d) {
         if (d.top < 1 || d.top > d.experts || d.top > 64) return "mixture of experts: 1 <= top <= min(experts, 64)";
     } else if (d.shared_ff > 0)
         return "a shared expert needs a mixture of experts";
-    if (d.mixer != GL3_MIX_ATTENTION && (d.rot_dims || d.v_unit_norm || d.v_rot || d.window > 0 || d.keep_first > 0))
-        return "rotary positions, value norm / rotation and windows belong to the attention mixer";
+    if (d.mixer != GL3_MIX_ATTENTION && (d.v_unit_norm || d.v_rot || d.window > 0 || d.keep_first > 0 || d.pool > 0 || d.qk_bias))
+        return "value norm / rotation, windows, pooled blocks and q / k / v biases belong to the attention mixer";
+    if (d.mixer != GL3_MIX_ATTENTION && d.mixer != GL3_MIX_MEMORY && d.rot_dims) return "rotary positions belong to the attention and matrix-memory mixers";
+    if (d.ff_act < 0 || d.ff_act > 1) return "ff_act must be 0 or 1";
     if (d.mixer == GL3_MIX_ATTENTION) {
         if (d.kv_heads < 1 || d.heads % d.kv_heads) return "attention: heads must be a multiple of kv_heads";
         if (d.dim < 1) return "attention: dim must be positive";
@@ -85,9 +90,19 @@ static const char* hy_check_layer(const gl3_layer_desc& d) {
         if ((d.rot_dims || d.v_rot) && !(d.rot_base > 0.f)) return "attention: rot_base must be positive";
         if (d.v_rot && (d.vdim & 1)) return "attention: rotated values need an even vdim";
         if (d.keep_first < 0) return "attention: keep_first must be >= 0";
+        if (d.qk_unit_norm < 0 || d.qk_unit_norm > 2 || d.softmax_sink < 0 || d.softmax_sink > 2) return "attention: qk_unit_norm and softmax_sink must be 0, 1 or 2";
+        if (d.pool < 0 || (d.pool > 0 && d.window <= 0)) return "attention: pooled blocks need a window";
+        if (d.pool > 0 && d.slope_log2 != 0.f) return "attention: pooled blocks have no distance term";
     } else if (d.mixer == GL3_MIX_LATENT) {
         if (d.dim < 1 || d.kv_rank < 1) return "latent attention: dim and kv_rank must be positive";
         if (d.kv_rank > 512) return "latent attention: kv_rank <= 512";
+    } else if (d.mixer == GL3_MIX_MEMORY) {
+        if (d.dim < 1 || d.dim > 2048) return "matrix memory: 1 <= dim <= 2048";
+        if (d.rot_dims < 0 || d.rot_dims > d.dim || (d.rot_dims & 1)) return "matrix memory: rot_dims must be even and at most dim";
+        if (d.rot_dims && !(d.rot_base > 0.f)) return "matrix memory: rot_base must be positive";
+        if (d.mem_gates != GL3_MEM_DECAY && d.mem_gates != GL3_MEM_EXP_GATES) return "matrix memory: unknown mem_gates";
+        if (d.mem_gates == GL3_MEM_DECAY && !d.mem_decay) return "matrix memory: a fixed decay needs mem_decay";
+        if (d.mem_gates == GL3_MEM_EXP_GATES && !(d.mem_gate_cap > 0.f)) return "matrix memory: mem_gate_cap must be positive";
     } else if (d.mixer == GL3_MIX_SSM) {
         if (d.state < 1 || d.state > 2048) return "ssm: 1 <= state <= 2048";
         if (d.groups < 1 || d.heads % d.groups) return "ssm: heads must be a multiple of groups";
@@ -108,8 +123,18 @@ int32_t gl3_hy_create(const gl3_model_desc* desc, gl3_ctx** out, std::string& er
     if (desc->dim < 1 || desc->vocab < 1 || desc->ctx < 1) { err = "layer-list family: dim, vocab and ctx must be positive"; return GL3_E_ARG; }
     if (desc->weight_type != GL3_TYPE_BF16 && desc->weight_type != GL3_TYPE_F32) { err = "layer-list family: weight_type must be GL3_TYPE_BF16 (or GL3_TYPE_F32)"; return GL3_E_UNSUPPORTED; }
     if (desc->tp_size > 1) { err = "layer-list family: tensor parallelism is not built"; return GL3_E_UNSUPPORTED; }
-    for (int l = 0; l < desc->n_layers; ++l)
-        if (const char* m = hy_check_layer(desc->layer_descs[l])) { err = "layer " + std::to_string(l) + ": " + m; return GL3_E_ARG; }
+    if (desc->parallel_block && (desc->streams > 0 || desc->side_dim || desc->depth_mix)) { err = "layer-list family: the parallel block needs the plain residual without token input and depth average"; return GL3_E_ARG; }
+    for (int l = 0; l < desc->n_layers; ++l) {
+        const gl3_layer_desc& ld = desc->layer_descs[l];
+        if (const char* m = hy_check_layer(ld)) { err = "layer " + std::to_string(l) + ": " + m; return GL3_E_ARG; }
+        if (desc->parallel_block && ld.experts > 0) { err = "layer-list family: the parallel block has a dense feed-forward"; return GL3_E_ARG; }
+        if (ld.beside) {
+            if (ld.beside->mixer == GL3_MIX_LATENT || ld.mixer == GL3_MIX_LATENT || ld.beside->mixer == GL3_MIX_SSM || ld.mixer == GL3_MIX_SSM) {
+                err = "layer " + std::to_string(l) + ": only attention and matrix-memory mixers can stand side by side"; return GL3_E_ARG;
+            }
+            if (const char* m = hy_check_layer(*ld.beside)) { err = "layer " + std::to_string(l) + ", second mixer: " + m; return GL3_E_ARG; }
+        }
+    }
     gl3_ctx* ctx = new gl3_ctx();
     ctx->d = *desc;
     ctx->d.layer_descs = nullptr;
@@ -117,6 +142,9 @@ int32_t gl3_hy_create(const gl3_model_desc* desc, gl3_ctx** out, std::string& er
     gl3_hybrid_state* h = ctx->hy = new gl3_hybrid_state();
     h->f32 = (desc->flags & GL3_FLAG_F32_COMPUTE) != 0;
     h->plain = desc->streams == 0;
+    h->parallel = desc->parallel_block != 0;
+    h->resid_mul = (h->parallel && desc->residual_scale != 0.f) ? desc->residual_scale : 1.f;
+    h->logit_mul = desc->logit_scale != 0.f ? desc->logit_scale : 1.f;
     h->emb_scale = desc->embedding_scale != 0.f ? desc->embedding_scale : 1.f;
     h->norm_offset = desc->norm_offset;
     h->side_dim = desc->side_dim; h->side_ld = hy_cdiv(std::max(1, desc->side_dim), 8) * 8;
@@ -139,12 +167,96 @@ int32_t gl3_hy_create(const gl3_model_desc* desc, gl3_ctx** out, std::string& er
     size_t slot = 0;
     int max_proj = 1, max_mix = W, max_ch = 1, max_inner = 1, max_hr = 1, max_hdv = 1, max_kx = 0, max_vx = 0, max_rz = 0, max_top = 0, max_eff = 0, max_e = 0;
     if (h->side_dim > 0) TRY(hy_alloc_mat(ctx, h->side_emb, V, desc->n_layers * h->side_dim, desc->n_layers * h->side_dim));
+    int max_heads = 1;
+    // one mixer's share of the layer: its offsets in the fused projection row (p0 = its first row) and in mixo / o (o0 = its first
+    // column), its vectors and tables, its part of the sequence slot
+    auto setup_mixer = [&](HyLayer& Ly, int p0, int o0) -> int32_t {
+        const gl3_layer_desc& d = Ly.d;
+        Ly.o0 = o0;
+        Ly.out_mul = d.out_scale != 0.f ? d.out_scale : 1.f;
+        max_heads = std::max(max_heads, d.heads);
+#define TRYM(x) do { int32_t r_ = (x); if (r_ != GL3_OK) return r_; } while (0)
+        // rotary tables, made in double: entry i turns by pos * base^(-2 i / dims) (q / k: divided by the position scaling)
+        auto table = [&](float** dst, int dims, double divide) -> int32_t {
+            std::vector<float> f(dims / 2);
+            for (int i = 0; i < dims / 2; ++i) f[i] = (float)(std::pow((double)d.rot_base, -2.0 * i / dims) / divide);
+            int32_t r_ = hy_alloc(ctx, dst, f.size() * 4);
+            if (r_ != GL3_OK) return r_;
+            return hipMemcpy(*dst, f.data(), f.size() * 4, hipMemcpyHostToDevice) == hipSuccess ? GL3_OK : GL3_E_HIP;
+        };
+        if (d.mixer == GL3_MIX_ATTENTION) {
+            Ly.q_off = p0; Ly.k_off = Ly.q_off + d.heads * d.dim; Ly.v_off = Ly.k_off + d.kv_heads * d.dim; Ly.g_off = Ly.v_off + d.kv_heads * d.vdim;
+            if (d.rot_dims > 0) TRYM(table(&Ly.rot_freq, d.rot_dims, d.rot_divide > 0.f ? (double)d.rot_divide : 1.0));
+            if (d.v_rot) TRYM(table(&Ly.vrot_freq, d.vdim, 1.0));
+            Ly.off_k = slot; slot += (size_t)C * d.kv_heads * d.dim;
+            Ly.off_v = slot; slot += (size_t)C * d.kv_heads * d.vdim;
+            if (d.pool > 0) {          // one pooled row per complete block of `pool` positions
+                Ly.off_pk = slot; slot += (size_t)(C / d.pool + 1) * d.kv_heads * d.dim;
+                Ly.off_pv = slot; slot += (size_t)(C / d.pool + 1) * d.kv_heads * d.vdim;
+            }
+            if (d.qk_unit_norm == 2) {
+                TRYM(hy_alloc(ctx, &Ly.qn, (size_t)d.heads * d.dim * 4));
+                TRYM(hy_alloc(ctx, &Ly.kn, (size_t)d.kv_heads * d.dim * 4));
+            }
+            if (d.softmax_sink == 2) TRYM(hy_alloc(ctx, &Ly.sink, (size_t)d.heads * 4));
+            max_hdv = std::max(max_hdv, d.heads * d.vdim);
+        } else if (d.mixer == GL3_MIX_LATENT) {
+            Ly.q_off = p0; Ly.c_off = Ly.q_off + d.heads * d.dim; Ly.g_off = Ly.c_off + d.kv_rank;
+            Ly.off_k = Ly.off_v = slot; slot += (size_t)C * d.kv_rank;
+            TRYM(hy_alloc(ctx, &Ly.lat_norm, (size_t)d.kv_rank * 4));
+            TRYM(hy_alloc(ctx, &Ly.wk, (size_t)d.heads * d.dim * d.kv_rank * 4));
+            TRYM(hy_alloc(ctx, &Ly.wv, (size_t)d.heads * d.vdim * d.kv_rank * 4));
+            TRYM(hy_alloc(ctx, &Ly.wvT, (size_t)d.heads * d.vdim * d.kv_rank * 4));
+            max_hr = std::max(max_hr, d.heads * d.kv_rank); max_hdv = std::max(max_hdv, std::max(d.heads * d.kv_rank, d.heads * d.vdim));
+            max_kx = std::max(max_kx, d.heads * d.dim); max_vx = std::max(max_vx, d.heads * d.vdim);
+        } else if (d.mixer == GL3_MIX_MEMORY) {
+            const bool eg = d.mem_gates == GL3_MEM_EXP_GATES;
+            Ly.d.kv_heads = d.heads;
+            Ly.q_off = p0; Ly.k_off = Ly.q_off + d.heads * d.dim; Ly.v_off = Ly.k_off + d.heads * d.dim; Ly.g_off = Ly.v_off + d.heads * d.vdim;
+            Ly.i_off = Ly.g_off + d.heads * d.vdim; Ly.f_off = Ly.i_off + d.heads;
+            if (d.rot_dims > 0) TRYM(table(&Ly.rot_freq, d.rot_dims, d.rot_divide > 0.f ? (double)d.rot_divide : 1.0));
+            const int P = d.vdim + (eg ? 1 : 0);             // exponential gates: one more state column carries the normaliser
+            Ly.off_state = slot; slot += (size_t)d.heads * d.dim * P;
+            if (eg) { Ly.off_m = slot; slot += (size_t)d.heads; }
+            else {
+                TRYM(hy_alloc(ctx, &Ly.decay, (size_t)d.heads * 4));
+                if (hipMemcpy(Ly.decay, d.mem_decay, (size_t)d.heads * 4, hipMemcpyHostToDevice) != hipSuccess) { ctx->err = "copy of mem_decay failed"; return GL3_E_HIP; }
+            }
+            if (d.mem_norm_weight) TRYM(hy_alloc(ctx, &Ly.ssm_norm, (size_t)d.heads * d.vdim * 4));
+            max_inner = std::max(max_inner, d.heads * P);
+        } else {
+            const int ch = hy_conv_ch(d), inner = d.heads * d.vdim;
+            Ly.off_state = slot; slot += (size_t)d.heads * d.state * d.vdim;
+            Ly.off_tail = slot; slot += (size_t)std::max(1, d.conv - 1) * ch;
+            TRYM(hy_alloc(ctx, &Ly.conv_w, (size_t)ch * d.conv * 4));
+            TRYM(hy_alloc(ctx, &Ly.conv_b, (size_t)ch * 4));
+            TRYM(hy_alloc(ctx, &Ly.dt_bias, (size_t)d.heads * 4));
+            TRYM(hy_alloc(ctx, &Ly.a_log, (size_t)d.heads * 4));
+            TRYM(hy_alloc(ctx, &Ly.dskip, (size_t)d.heads * 4));
+            TRYM(hy_alloc(ctx, &Ly.ssm_norm, (size_t)inner * 4));
+            max_ch = std::max(max_ch, ch); max_inner = std::max(max_inner, inner);
+        }
+#undef TRYM
+        Ly.d.mem_decay = nullptr;          // the caller's array is not kept
+        Ly.d.beside = nullptr;
+        return GL3_OK;
+    };
     for (int l = 0; l < desc->n_layers; ++l) {
         HyLayer& Ly = h->L[l];
         const gl3_layer_desc& d = Ly.d = desc->layer_descs[l];
-        const int np = hy_proj_rows(d), mo = hy_mix_out(d);
+        const gl3_layer_desc* bd = d.beside;
+        if (bd) {
+            Ly.side = new HyLayer();
+            Ly.side->d = *bd;
+            Ly.side->d.ff = 0; Ly.side->d.experts = 0; Ly.side->d.shared_ff = 0;
+        }
+        const int np1 = hy_proj_rows(d), mo1 = hy_mix_out(d);
+        const int np = np1 + (bd ? hy_proj_rows(*bd) : 0), mo = mo1 + (bd ? hy_mix_out(*bd) : 0);
+        const bool bias = hy_has_bias(d) || (bd && hy_has_bias(*bd));
+        Ly.mo_total = mo;
         TRY(hy_alloc_mat(ctx, Ly.proj, np, W, W));
         TRY(hy_alloc_mat(ctx, Ly.o, W, mo, mo));
+        if (bias) TRY(hy_alloc(ctx, &Ly.pbias, (size_t)np * 4));
         TRY(hy_alloc(ctx, &Ly.norm1, (size_t)W * 4));
         for (int q = 0; q < (d.ff > 0 ? 2 : 1) && !h->plain; ++q) {
             TRY(hy_alloc(ctx, &Ly.hc[q][0], (size_t)S * 4));
@@ -152,45 +264,14 @@ int32_t gl3_hy_create(const gl3_model_desc* desc, gl3_ctx** out, std::string& er
             TRY(hy_alloc(ctx, &Ly.hc[q][2], (size_t)S * S * 4));
         }
         max_proj = std::max(max_proj, np); max_mix = std::max(max_mix, mo);
-        if (d.mixer == GL3_MIX_ATTENTION) {
-            Ly.q_off = 0; Ly.k_off = d.heads * d.dim; Ly.v_off = Ly.k_off + d.kv_heads * d.dim; Ly.g_off = Ly.v_off + d.kv_heads * d.vdim;
-            // rotary tables, made in double: entry i turns by pos * base^(-2 i / dims) (q / k: divided by the position scaling)
-            auto table = [&](float** dst, int dims, double divide) -> int32_t {
-                std::vector<float> f(dims / 2);
-                for (int i = 0; i < dims / 2; ++i) f[i] = (float)(std::pow((double)d.rot_base, -2.0 * i / dims) / divide);
-                int32_t r_ = hy_alloc(ctx, dst, f.size() * 4);
-                if (r_ != GL3_OK) return r_;
-                return hipMemcpy(*dst, f.data(), f.size() * 4, hipMemcpyHostToDevice) == hipSuccess ? GL3_OK : GL3_E_HIP;
-            };
-            if (d.rot_dims > 0) TRY(table(&Ly.rot_freq, d.rot_dims, d.rot_divide > 0.f ? (double)d.rot_divide : 1.0));
-            if (d.v_rot) TRY(table(&Ly.vrot_freq, d.vdim, 1.0));
-            Ly.off_k = slot; slot += (size_t)C * d.kv_heads * d.dim;
-            Ly.off_v = slot; slot += (size_t)C * d.kv_heads * d.vdim;
-            max_hdv = std::max(max_hdv, d.heads * d.vdim);
-        } else if (d.mixer == GL3_MIX_LATENT) {
-            Ly.q_off = 0; Ly.c_off = d.heads * d.dim; Ly.g_off = Ly.c_off + d.kv_rank;
-            Ly.off_k = Ly.off_v = slot; slot += (size_t)C * d.kv_rank;
-            TRY(hy_alloc(ctx, &Ly.lat_norm, (size_t)d.kv_rank * 4));
-            TRY(hy_alloc(ctx, &Ly.wk, (size_t)d.heads * d.dim * d.kv_rank * 4));
-            TRY(hy_alloc(ctx, &Ly.wv, (size_t)d.heads * d.vdim * d.kv_rank * 4));
-            TRY(hy_alloc(ctx, &Ly.wvT, (size_t)d.heads * d.vdim * d.kv_rank * 4));
-            max_hr = std::max(max_hr, d.heads * d.kv_rank); max_hdv = std::max(max_hdv, std::max(d.heads * d.kv_rank, d.heads * d.vdim));
-            max_kx = std::max(max_kx, d.heads * d.dim); max_vx = std::max(max_vx, d.heads * d.vdim);
-        } else {
-            const int ch = hy_conv_ch(d), inner = d.heads * d.vdim;
-            Ly.off_state = slot; slot += (size_t)d.heads * d.state * d.vdim;
-            Ly.off_tail = slot; slot += (size_t)std::max(1, d.conv - 1) * ch;
-            TRY(hy_alloc(ctx, &Ly.conv_w, (size_t)ch * d.conv * 4));
-            TRY(hy_alloc(ctx, &Ly.conv_b, (size_t)ch * 4));
-            TRY(hy_alloc(ctx, &Ly.dt_bias, (size_t)d.heads * 4));
-            TRY(hy_alloc(ctx, &Ly.a_log, (size_t)d.heads * 4));
-            TRY(hy_alloc(ctx, &Ly.dskip, (size_t)d.heads * 4));
-            TRY(hy_alloc(ctx, &Ly.ssm_norm, (size_t)inner * 4));
-            max_ch = std::max(max_ch, ch); max_inner = std::max(max_inner, inner);
+        TRY(setup_mixer(Ly, 0, 0));
+        if (Ly.side) {
+            Ly.side->pbias = Ly.pbias; Ly.side->mo_total = mo;
+            TRY(setup_mixer(*Ly.side, np1, mo1));
         }
         Ly.dense_ff = d.experts > 0 ? d.shared_ff : d.ff;
         Ly.dense_limit = d.experts > 0 ? d.shared_limit : d.ff_limit;
-        if (d.ff > 0) TRY(hy_alloc(ctx, &Ly.norm2, (size_t)W * 4));
+        if (d.ff > 0 && !h->parallel) TRY(hy_alloc(ctx, &Ly.norm2, (size_t)W * 4));
         if (Ly.dense_ff > 0) {
             Ly.ff_pad = hy_cdiv(Ly.dense_ff, 32) * 32;
             TRY(hy_alloc_mat(ctx, Ly.gu, 2 * Ly.ff_pad, W, W));
@@ -217,7 +298,10 @@ int32_t gl3_hy_create(const gl3_model_desc* desc, gl3_ctx** out, std::string& er
     TRY(hy_alloc(ctx, &h->X, (size_t)S * mb * W * 4));
     TRY(hy_alloc(ctx, &h->h, (size_t)mb * W * es));
     TRY(hy_alloc(ctx, &h->proj, (size_t)mb * max_proj * 4));
-    TRY(hy_alloc(ctx, &h->y, (size_t)HY_KSPLIT * mb * W * 4));          // K-split partial sums of the output / down projections
+    TRY(hy_alloc(ctx, &h->y, (size_t)HY_YPARTS * mb * W * 4));          // K-split partial sums of the output / down projections
+    h->max_heads = max_heads;
+    TRY(hy_alloc(ctx, &h->gates, (size_t)3 * mb * max_heads * 4));
+    TRY(hy_alloc(ctx, &h->rowr, (size_t)2 * mb * 4));
     TRY(hy_alloc(ctx, &h->mixo, (size_t)mb * max_mix * es));
     TRY(hy_alloc(ctx, &h->conv, (size_t)mb * max_ch * 4));
     TRY(hy_alloc(ctx, &h->ssm_y, (size_t)mb * max_inner * 4));
@@ -229,11 +313,7 @@ int32_t gl3_hy_create(const gl3_model_desc* desc, gl3_ctx** out, std::string& er
     }
     h->part_rows = std::max<size_t>(mb, 16 * 128);         // (token, split) pairs: a portion at one split, or 16 decode tokens at 128
     TRY(hy_alloc(ctx, &h->part_acc, h->part_rows * max_hdv * 4));
-    {
-        int max_h = 1;
-        for (auto& Ly : h->L) max_h = std::max(max_h, Ly.d.heads);
-        TRY(hy_alloc(ctx, &h->part_ml, h->part_rows * max_h * 2 * 4));
-    }
+    TRY(hy_alloc(ctx, &h->part_ml, h->part_rows * max_heads * 2 * 4));
     if (h->depth) TRY(hy_alloc(ctx, &h->hist, (size_t)(desc->n_layers + 1) * mb * W * 4));
     if (h->side_dim > 0) {
         TRY(hy_alloc(ctx, &h->xb, (size_t)mb * W * es));
@@ -294,13 +374,19 @@ void gl3_hy_destroy(gl3_ctx* ctx) {
     auto hf = [](void* p) { if (p) hipHostFree(p); };
     f(h->emb.w); f(h->head.w); f(h->final_norm);
     for (auto& L : h->L) {
-        f(L.proj.w); f(L.o.w); f(L.gu.w); f(L.down.w); f(L.norm1); f(L.norm2);
+        f(L.proj.w); f(L.o.w); f(L.gu.w); f(L.down.w); f(L.norm1); f(L.norm2); f(L.pbias);
         for (auto& q : L.hc) for (float* p : q) f(p);
-        f(L.lat_norm); f(L.wk); f(L.wv); f(L.wvT); f(L.conv_w); f(L.conv_b); f(L.dt_bias); f(L.a_log); f(L.dskip); f(L.ssm_norm);
-        f(L.router.w); f(L.egu.w); f(L.edown.w); f(L.depth_mix); f(L.side_gate.w); f(L.side_proj.w); f(L.side_norm); f(L.rot_freq); f(L.vrot_freq);
+        for (HyLayer* M : {&L, L.side}) {
+            if (!M) continue;
+            f(M->lat_norm); f(M->wk); f(M->wv); f(M->wvT); f(M->conv_w); f(M->conv_b); f(M->dt_bias); f(M->a_log); f(M->dskip); f(M->ssm_norm);
+            f(M->rot_freq); f(M->vrot_freq); f(M->qn); f(M->kn); f(M->sink); f(M->decay);
+        }
+        delete L.side;
+        L.side = nullptr;
+        f(L.router.w); f(L.egu.w); f(L.edown.w); f(L.depth_mix); f(L.side_gate.w); f(L.side_proj.w); f(L.side_norm);
     }
     f(h->side_emb.w); f(h->sgz); f(h->hist); f(h->side_z); f(h->moe_z); f(h->wsel); f(h->eout); f(h->xb); f(h->side_g); f(h->ea); f(h->eact); f(h->sel); f(h->pair_row); f(h->tiles); f(h->ntiles);
-    f(h->slots); f(h->X); f(h->h); f(h->proj); f(h->y); f(h->mixo); f(h->conv); f(h->ssm_y); f(h->qa); f(h->oc); f(h->kx); f(h->vx); f(h->part_acc); f(h->part_ml);
+    f(h->slots); f(h->X); f(h->h); f(h->proj); f(h->y); f(h->mixo); f(h->conv); f(h->ssm_y); f(h->qa); f(h->oc); f(h->kx); f(h->vx); f(h->part_acc); f(h->part_ml); f(h->gates); f(h->rowr);
     f(h->xw); f(h->logits); f(h->taps); f(h->ones); f(h->dyn);
     hf(h->h_dyn); hf(h->h_logits);
     if (ctx->logits == h->logits) ctx->logits = nullptr;
@@ -330,28 +416,28 @@ static int32_t hy_put_vec(gl3_ctx* ctx, float* dst, size_t n, const void* host, 
     HY_HIP(hipMemcpy(dst, f.data(), n * 4, hipMemcpyHostToDevice));
     return GL3_OK;
 }
-// rows x k source -> rows dst_row0 .. of m.  block32 = 1 / 2: source row r goes to row (r / 32) 64 + r % 32 (+ 32 for 2)
-static int32_t hy_put_rows(gl3_ctx* ctx, HyMat& m, int dst_row0, int rows, int k, const void* host, uint64_t bytes, int type, int block32) {
+// rows x k source -> rows dst_row0 .., columns dst_col0 .. dst_col0 + k - 1 of m (the matrix's other columns keep what they hold).
+// block32 = 1 / 2: source row r goes to row (r / 32) 64 + r % 32 (+ 32 for 2)
+static int32_t hy_put_rows(gl3_ctx* ctx, HyMat& m, int dst_row0, int rows, int k, const void* host, uint64_t bytes, int type, int block32, int dst_col0 = 0) {
     const bool f32 = ctx->hy->f32;
     const size_t es = f32 ? 4 : 2, n = (size_t)rows * k;
     if ((type != GL3_TYPE_BF16 && type != GL3_TYPE_F32) || bytes != n * (type == GL3_TYPE_BF16 ? 2 : 4)) GL3_FAIL(GL3_E_ARG, "tensor size or type mismatch");
-    if (k > m.ld || k != m.k) GL3_FAIL(GL3_E_ARG, "tensor row length mismatch");
-    std::vector<uint8_t> img((size_t)rows * m.ld * es, 0);
-    for (int r = 0; r < rows; ++r)
-        for (int c = 0; c < k; ++c) {
-            const size_t si = (size_t)r * k + c, di = (size_t)r * m.ld + c;
-            if (f32) ((float*)img.data())[di] = type == GL3_TYPE_BF16 ? hy_bf16_to_f32(((const uint16_t*)host)[si]) : ((const float*)host)[si];
-            else ((uint16_t*)img.data())[di] = type == GL3_TYPE_BF16 ? ((const uint16_t*)host)[si] : hy_f32_to_bf16(((const float*)host)[si]);
-        }
-    const size_t rb = (size_t)m.ld * es;
+    if (dst_col0 < 0 || dst_col0 + k > m.k) GL3_FAIL(GL3_E_ARG, "tensor row length mismatch");
+    std::vector<uint8_t> img(n * es, 0);
+    for (size_t i = 0; i < n; ++i) {
+        if (f32) ((float*)img.data())[i] = type == GL3_TYPE_BF16 ? hy_bf16_to_f32(((const uint16_t*)host)[i]) : ((const float*)host)[i];
+        else ((uint16_t*)img.data())[i] = type == GL3_TYPE_BF16 ? ((const uint16_t*)host)[i] : hy_f32_to_bf16(((const float*)host)[i]);
+    }
+    const size_t rb = (size_t)m.ld * es, sb = (size_t)k * es;
+    uint8_t* base = (uint8_t*)m.w + (size_t)dst_col0 * es;
     if (!block32) {
         if (dst_row0 + rows > m.rows) GL3_FAIL(GL3_E_ARG, "tensor has too many rows");
-        HY_HIP(hipMemcpy((uint8_t*)m.w + (size_t)dst_row0 * rb, img.data(), (size_t)rows * rb, hipMemcpyHostToDevice));
+        HY_HIP(hipMemcpy2D(base + (size_t)dst_row0 * rb, rb, img.data(), sb, sb, rows, hipMemcpyHostToDevice));
     } else {
         for (int r0 = 0; r0 < rows; r0 += 32) {
             const int nr = std::min(32, rows - r0), dr = dst_row0 + (r0 / 32) * 64 + (block32 == 2 ? 32 : 0);
             if (dr + nr > m.rows) GL3_FAIL(GL3_E_ARG, "tensor has too many rows");
-            HY_HIP(hipMemcpy((uint8_t*)m.w + (size_t)dr * rb, img.data() + (size_t)r0 * rb, (size_t)nr * rb, hipMemcpyHostToDevice));
+            HY_HIP(hipMemcpy2D(base + (size_t)dr * rb, rb, img.data() + (size_t)r0 * sb, sb, sb, nr, hipMemcpyHostToDevice));
         }
     }
     return GL3_OK;
@@ -375,22 +461,38 @@ int32_t gl3_hy_upload(gl3_ctx* ctx, int32_t id, int32_t layer, const void* host,
         if (r == GL3_OK) h->have |= 1ull << id;
         return r;
     }
+    const bool beside = layer >= 0 && (layer & GL3_LAYER_BESIDE);
+    if (beside) layer &= ~GL3_LAYER_BESIDE;
     if (layer < 0 || layer >= (int)h->L.size()) GL3_FAIL(GL3_E_ARG, "layer out of range");
-    HyLayer& L = h->L[layer];
+    HyLayer& L0 = h->L[layer];                       // the layer: its fused projection, output projection and feed-forward
+    if (beside && !L0.side) GL3_FAIL(GL3_E_ARG, "layer " + std::to_string(layer) + " has no second mixer");
+    HyLayer& L = beside ? *L0.side : L0;             // the mixer the tensor belongs to
     const gl3_layer_desc& d = L.d;
-    const bool att = d.mixer == GL3_MIX_ATTENTION, lat = d.mixer == GL3_MIX_LATENT, ssm = d.mixer == GL3_MIX_SSM;
+    const bool att = d.mixer == GL3_MIX_ATTENTION, lat = d.mixer == GL3_MIX_LATENT, ssm = d.mixer == GL3_MIX_SSM, mem = d.mixer == GL3_MIX_MEMORY;
+    const bool memg = mem && d.mem_gates == GL3_MEM_EXP_GATES;
     const int mo = hy_mix_out(d);
+    HyMat& proj = L0.proj;
     const size_t tes = type == GL3_TYPE_BF16 ? 2 : 4;          // bytes per element of the source
     std::vector<float> f;
     switch (id) {
-        case GL3_T_ATTN_NORM: r = hy_put_vec(ctx, L.norm1, W, host, bytes, type, h->norm_offset); break;
-        case GL3_T_FFN_NORM: if (d.ff > 0) r = hy_put_vec(ctx, L.norm2, W, host, bytes, type, h->norm_offset); break;
-        case GL3_T_WQ: if (att || lat) r = hy_put_rows(ctx, L.proj, L.q_off, d.heads * d.dim, W, host, bytes, type, 0); break;
-        case GL3_T_WK: if (att) r = hy_put_rows(ctx, L.proj, L.k_off, d.kv_heads * d.dim, W, host, bytes, type, 0); break;
-        case GL3_T_WV: if (att) r = hy_put_rows(ctx, L.proj, L.v_off, d.kv_heads * d.vdim, W, host, bytes, type, 0); break;
-        case GL3_T_ATTN_GATE: if ((att || lat) && d.out_gate) r = hy_put_rows(ctx, L.proj, L.g_off, hy_gate_rows(d), W, host, bytes, type, 0); break;
-        case GL3_T_WO: r = hy_put_rows(ctx, L.o, 0, W, mo, host, bytes, type, 0); break;
-        case GL3_T_KV_DOWN: if (lat) r = hy_put_rows(ctx, L.proj, L.c_off, d.kv_rank, W, host, bytes, type, 0); break;
+        case GL3_T_ATTN_NORM: if (!beside) r = hy_put_vec(ctx, L.norm1, W, host, bytes, type, h->norm_offset); break;
+        case GL3_T_FFN_NORM: if (d.ff > 0 && L.norm2) r = hy_put_vec(ctx, L.norm2, W, host, bytes, type, h->norm_offset); break;
+        case GL3_T_WQ: if (att || lat || mem) r = hy_put_rows(ctx, proj, L.q_off, d.heads * d.dim, W, host, bytes, type, 0); break;
+        case GL3_T_WK: if (att || mem) r = hy_put_rows(ctx, proj, L.k_off, d.kv_heads * d.dim, W, host, bytes, type, 0); break;
+        case GL3_T_WV: if (att || mem) r = hy_put_rows(ctx, proj, L.v_off, d.kv_heads * d.vdim, W, host, bytes, type, 0); break;
+        case GL3_T_ATTN_GATE: if (((att || lat) && d.out_gate) || mem) r = hy_put_rows(ctx, proj, L.g_off, hy_gate_rows(d), W, host, bytes, type, 0); break;
+        case GL3_T_WO: r = hy_put_rows(ctx, L0.o, 0, W, mo, host, bytes, type, 0, L.o0); break;
+        case GL3_T_BQ: if (att && d.qk_bias) r = hy_put_vec(ctx, L.pbias + L.q_off, (size_t)d.heads * d.dim, host, bytes, type); break;
+        case GL3_T_BK: if (att && d.qk_bias) r = hy_put_vec(ctx, L.pbias + L.k_off, (size_t)d.kv_heads * d.dim, host, bytes, type); break;
+        case GL3_T_BV: if (att && d.qk_bias) r = hy_put_vec(ctx, L.pbias + L.v_off, (size_t)d.kv_heads * d.vdim, host, bytes, type); break;
+        case GL3_T_ATTN_Q_NORM: if (att && d.qk_unit_norm == 2) r = hy_put_vec(ctx, L.qn, (size_t)d.heads * d.dim, host, bytes, type); break;
+        case GL3_T_ATTN_K_NORM: if (att && d.qk_unit_norm == 2) r = hy_put_vec(ctx, L.kn, (size_t)d.kv_heads * d.dim, host, bytes, type); break;
+        case GL3_T_ATTN_SINK: if (att && d.softmax_sink == 2) r = hy_put_vec(ctx, L.sink, d.heads, host, bytes, type); break;
+        case GL3_T_MEM_IGATE: if (memg) r = hy_put_rows(ctx, proj, L.i_off, d.heads, W, host, bytes, type, 0); break;
+        case GL3_T_MEM_FGATE: if (memg) r = hy_put_rows(ctx, proj, L.f_off, d.heads, W, host, bytes, type, 0); break;
+        case GL3_T_MEM_IGATE_BIAS: if (memg) r = hy_put_vec(ctx, L.pbias + L.i_off, d.heads, host, bytes, type); break;
+        case GL3_T_MEM_FGATE_BIAS: if (memg) r = hy_put_vec(ctx, L.pbias + L.f_off, d.heads, host, bytes, type); break;
+        case GL3_T_KV_DOWN: if (lat) r = hy_put_rows(ctx, proj, L.c_off, d.kv_rank, W, host, bytes, type, 0); break;
         case GL3_T_KV_DOWN_NORM: if (lat) r = hy_put_vec(ctx, L.lat_norm, d.kv_rank, host, bytes, type); break;
         case GL3_T_K_UP: if (lat) r = hy_put_vec(ctx, L.wk, (size_t)d.heads * d.dim * d.kv_rank, host, bytes, type); break;
         case GL3_T_V_UP:
@@ -406,13 +508,13 @@ int32_t gl3_hy_upload(gl3_ctx* ctx, int32_t id, int32_t layer, const void* host,
                 r = GL3_OK;
             }
             break;
-        case GL3_T_SSM_IN: if (ssm) r = hy_put_rows(ctx, L.proj, 0, hy_proj_rows(d), W, host, bytes, type, 0); break;
+        case GL3_T_SSM_IN: if (ssm) r = hy_put_rows(ctx, proj, L.q_off, hy_proj_rows(d), W, host, bytes, type, 0); break;
         case GL3_T_SSM_CONV: if (ssm) r = hy_put_vec(ctx, L.conv_w, (size_t)hy_conv_ch(d) * d.conv, host, bytes, type); break;
         case GL3_T_SSM_CONV_BIAS: if (ssm) r = hy_put_vec(ctx, L.conv_b, hy_conv_ch(d), host, bytes, type); break;
         case GL3_T_SSM_DT_BIAS: if (ssm) r = hy_put_vec(ctx, L.dt_bias, d.heads, host, bytes, type); break;
         case GL3_T_SSM_A_LOG: if (ssm) r = hy_put_vec(ctx, L.a_log, d.heads, host, bytes, type); break;
         case GL3_T_SSM_D: if (ssm) r = hy_put_vec(ctx, L.dskip, d.heads, host, bytes, type); break;
-        case GL3_T_SSM_NORM: if (ssm) r = hy_put_vec(ctx, L.ssm_norm, mo, host, bytes, type); break;
+        case GL3_T_SSM_NORM: if (ssm || (mem && d.mem_norm_weight)) r = hy_put_vec(ctx, L.ssm_norm, mo, host, bytes, type); break;
         case GL3_T_W1: if (L.dense_ff > 0) r = hy_put_rows(ctx, L.gu, 0, L.dense_ff, W, host, bytes, type, 1); break;
         case GL3_T_W3: if (L.dense_ff > 0) r = hy_put_rows(ctx, L.gu, 0, L.dense_ff, W, host, bytes, type, 2); break;
         case GL3_T_W2:
@@ -462,18 +564,28 @@ int32_t gl3_hy_upload(gl3_ctx* ctx, int32_t id, int32_t layer, const void* host,
     return r;
 }
 
-static uint64_t hy_needed(const gl3_hybrid_state* h, const gl3_layer_desc& d) {
-    uint64_t m = (1ull << GL3_T_ATTN_NORM) | (1ull << GL3_T_WO);
+// tensors of one mixer (second = the mixer beside the layer's first: it has no norm, tables or feed-forward of its own)
+static uint64_t hy_needed(const gl3_hybrid_state* h, const gl3_layer_desc& d, bool second = false) {
+    uint64_t m = 1ull << GL3_T_WO;
+    if (d.mixer == GL3_MIX_ATTENTION) m |= (1ull << GL3_T_WQ) | (1ull << GL3_T_WK) | (1ull << GL3_T_WV);
+    if (d.mixer == GL3_MIX_ATTENTION && d.qk_bias) m |= (1ull << GL3_T_BQ) | (1ull << GL3_T_BK) | (1ull << GL3_T_BV);
+    if (d.mixer == GL3_MIX_ATTENTION && d.qk_unit_norm == 2) m |= (1ull << GL3_T_ATTN_Q_NORM) | (1ull << GL3_T_ATTN_K_NORM);
+    if (d.mixer == GL3_MIX_ATTENTION && d.softmax_sink == 2) m |= 1ull << GL3_T_ATTN_SINK;
+    if (d.mixer == GL3_MIX_MEMORY) m |= (1ull << GL3_T_WQ) | (1ull << GL3_T_WK) | (1ull << GL3_T_WV) | (1ull << GL3_T_ATTN_GATE);
+    if (d.mixer == GL3_MIX_MEMORY && d.mem_norm_weight) m |= 1ull << GL3_T_SSM_NORM;
+    if (d.mixer == GL3_MIX_MEMORY && d.mem_gates == GL3_MEM_EXP_GATES)
+        m |= (1ull << GL3_T_MEM_IGATE) | (1ull << GL3_T_MEM_FGATE) | (1ull << GL3_T_MEM_IGATE_BIAS) | (1ull << GL3_T_MEM_FGATE_BIAS);
+    if (second) return m;
+    m |= 1ull << GL3_T_ATTN_NORM;
     if (!h->plain) m |= (1ull << GL3_T_HC1_IN) | (1ull << GL3_T_HC1_OUT) | (1ull << GL3_T_HC1_MIX);
     if (h->depth) m |= 1ull << GL3_T_DEPTH_MIX;
     if (h->side_dim > 0) m |= (1ull << GL3_T_SIDE_GATE) | (1ull << GL3_T_SIDE_PROJ) | (1ull << GL3_T_SIDE_NORM);
-    if (d.mixer == GL3_MIX_ATTENTION) m |= (1ull << GL3_T_WQ) | (1ull << GL3_T_WK) | (1ull << GL3_T_WV);
     if (d.mixer == GL3_MIX_LATENT) m |= (1ull << GL3_T_WQ) | (1ull << GL3_T_KV_DOWN) | (1ull << GL3_T_KV_DOWN_NORM) | (1ull << GL3_T_K_UP) | (1ull << GL3_T_V_UP);
-    if (d.mixer != GL3_MIX_SSM && d.out_gate) m |= 1ull << GL3_T_ATTN_GATE;
+    if ((d.mixer == GL3_MIX_ATTENTION || d.mixer == GL3_MIX_LATENT) && d.out_gate) m |= 1ull << GL3_T_ATTN_GATE;
     if (d.mixer == GL3_MIX_SSM)
         m |= (1ull << GL3_T_SSM_IN) | (1ull << GL3_T_SSM_CONV) | (1ull << GL3_T_SSM_CONV_BIAS) | (1ull << GL3_T_SSM_DT_BIAS) | (1ull << GL3_T_SSM_A_LOG) |
              (1ull << GL3_T_SSM_D) | (1ull << GL3_T_SSM_NORM);
-    if (d.ff > 0) m |= 1ull << GL3_T_FFN_NORM;
+    if (d.ff > 0 && !h->parallel) m |= 1ull << GL3_T_FFN_NORM;
     if (d.ff > 0 && !h->plain) m |= (1ull << GL3_T_HC2_IN) | (1ull << GL3_T_HC2_OUT) | (1ull << GL3_T_HC2_MIX);
     if (d.experts > 0) m |= (1ull << GL3_T_FFN_GATE_INP) | (1ull << GL3_T_FFN_GATE_EXPS) | (1ull << GL3_T_FFN_UP_EXPS) | (1ull << GL3_T_FFN_DOWN_EXPS);
     if (d.experts > 0 && d.shared_ff > 0) m |= 1ull << GL3_T_FFN_GATE_INP_SHEXP;
@@ -491,6 +603,16 @@ int32_t gl3_hy_finalize(gl3_ctx* ctx) {
     for (size_t l = 0; l < h->L.size(); ++l) {
         const uint64_t need = hy_needed(h, h->L[l].d);
         if ((h->L[l].have & need) != need) GL3_FAIL(GL3_E_STATE, "layer " + std::to_string(l) + ": missing tensors");
+        if (h->L[l].side) {
+            const uint64_t need2 = hy_needed(h, h->L[l].side->d, true);
+            if ((h->L[l].side->have & need2) != need2) GL3_FAIL(GL3_E_STATE, "layer " + std::to_string(l) + ", second mixer: missing tensors");
+        }
+    }
+    if (h->logit_mul != 1.f) {          // the logits' multiplier rides on the final norm's weight
+        std::vector<float> w(h->W);
+        HY_HIP(hipMemcpy(w.data(), h->final_norm, (size_t)h->W * 4, hipMemcpyDeviceToHost));
+        for (float& v : w) v *= h->logit_mul;
+        HY_HIP(hipMemcpy(h->final_norm, w.data(), (size_t)h->W * 4, hipMemcpyHostToDevice));
     }
     HY_HIP(hipDeviceSynchronize());
     ctx->finalized = true;
@@ -498,6 +620,8 @@ int32_t gl3_hy_finalize(gl3_ctx* ctx) {
 }
 
 // ---- launches -----------------------------------------------------------------------------------------------------------------------
+// activation of the layer's dense feed-forward (in a mixture of experts: of the shared expert)
+static HyGlu hy_ff_glu(const HyLayer& L) { return HyGlu{L.dense_limit, L.d.ff_alpha, L.d.ff_shift, nullptr, nullptr, 0, 0, L.d.ff_act}; }
 // parts != null: C has room for HY_KSPLIT copies and the caller sums them (the streams kernel does); *parts = copies written
 template <typename T>
 static void hy_gemm(gl3_ctx* ctx, const T* A, int lda, const HyMat& w, int M, float* C, int ldc, bool glu, T* act, int ld_act, HyGlu gp, int* parts = nullptr, int max_parts = HY_KSPLIT) {
@@ -574,7 +698,7 @@ static HyAttnPlan hy_attn_plan(int rows, int dk, int dv, bool shared_kv) {
 }
 
 static int32_t hy_attention(gl3_ctx* ctx, const float* q, int ldq, const float* kc, const float* vc, int H, int G, int dk, int dv, float scale, float slope_log2,
-                            int n, int pos0, int* nsplit_out, bool in_slot = true, int window = 0, int keep = 0) {
+                            int n, int pos0, int* nsplit_out, bool in_slot = true, int window = 0, int keep = 0, const float* pk = nullptr, const float* pv = nullptr, int pool = 0) {
     gl3_hybrid_state* h = ctx->hy;
     const bool shared_kv = kc == vc && dk == dv;
     HyAttnPlan p = hy_attn_plan(n * (H / G), dk, dv, shared_kv);
@@ -583,12 +707,14 @@ static int32_t hy_attention(gl3_ctx* ctx, const float* q, int ldq, const float* 
     if (n <= 16) {
         int tiles = hy_cdiv(pos0 + n, p.kt);
         if (window > 0) tiles = std::min<long>(tiles, hy_cdiv(keep, p.kt) + ((long)window + n) / p.kt + 2);      // kept first keys + the window's tiles
+        if (pool > 0) tiles += hy_cdiv(std::max(0, pos0 + n - window) / pool, p.kt);                               // + the tiles of pooled rows
         nsplit = std::min(128, std::max(1, tiles));
     }
     if ((size_t)n * nsplit > h->part_rows) nsplit = std::max<size_t>(1, h->part_rows / n);
     HyAttnArgs a;
     a.q = q; a.ldq = ldq; a.kc = kc; a.vc = vc; a.slot_stride = in_slot ? h->slot_floats : 0; a.H = H; a.G = G; a.dk = dk; a.dv = dv; a.scale = scale; a.slope_log2 = slope_log2;
     a.dyn = h->dyn; a.n = n; a.nsplit = nsplit; a.part_acc = h->part_acc; a.part_ml = h->part_ml; a.kt = p.kt; a.shared_kv = shared_kv ? 1 : 0; a.window = window; a.keep = keep;
+    a.pk = pk; a.pv = pv; a.pool = pool;
     const dim3 grid((unsigned)hy_cdiv(n * (H / G), 4 * p.rw) * G, 1, nsplit);
 #define HY_AT(RW, DVL) hipLaunchKernelGGL((hy_attn_kernel<RW, DVL>), grid, dim3(256), p.smem, ctx->stream, a)
 #define HY_AT_RW(RW) do { if (p.dvl == 1) HY_AT(RW, 1); else if (p.dvl == 2) HY_AT(RW, 2); else if (p.dvl == 4) HY_AT(RW, 4); else HY_AT(RW, 8); } while (0)
@@ -600,27 +726,74 @@ static int32_t hy_attention(gl3_ctx* ctx, const float* q, int ldq, const float* 
     return GL3_OK;
 }
 
+// The recurrence kernel: a column's states over NG lanes x NL registers: NL = 16 (32 for more than 1024 states, 8 / 4 for very small
+// ones), NG a power of two; tokens staged per round: what fits 48 KB of LDS, at most 32.  Fills in a.NG and a.TB.
+static void hy_scan(gl3_ctx* ctx, HyScanArgs& a) {
+    const int NL = a.N > 1024 ? 32 : a.N > 8 ? 16 : a.N > 4 ? 8 : 4;
+    int NG = 1;
+    while (NG * NL < a.N) NG *= 2;
+    const int cols = 4 * (64 / NG), Ns = NG * NL;
+    int TB = (int)(48 * 1024 / ((2 * (size_t)Ns + cols + 258) * 4));
+    TB = std::max(1, std::min(32, TB));
+    const size_t smem = ((size_t)TB * (2 * Ns + cols + 256) + 2 * TB) * 4;
+    a.NG = NG; a.TB = TB;
+    const dim3 grid(hy_cdiv(a.P, cols), a.heads);
+#define HY_SCAN(NLT) hipLaunchKernelGGL((hy_ssm_scan_kernel<NLT>), grid, dim3(256), smem, ctx->stream, a)
+    if (NL == 4) HY_SCAN(4); else if (NL == 8) HY_SCAN(8); else if (NL == 16) HY_SCAN(16); else HY_SCAN(32);
+#undef HY_SCAN
+}
+
+// One mixer of a layer on the n rows of the fused projection in h->proj (row stride np): its heads land in mixo (row stride ldo) from
+// column L.o0 on, multiplied by L.out_mul.
 template <typename T>
-static int32_t hy_mixer(gl3_ctx* ctx, HyLayer& L, int n, int pos0, int seq) {
+static int32_t hy_mixer_core(gl3_ctx* ctx, HyLayer& L, int np, int ldo, int n, int pos0, int seq) {
     gl3_hybrid_state* h = ctx->hy;
     const gl3_layer_desc& d = L.d;
     hipStream_t st = ctx->stream;
     const float eps = ctx->d.rms_eps;
-    const int np = L.proj.rows;
-    T* hin = (T*)h->h;
-    T* mixo = (T*)h->mixo;
-    hy_gemm<T>(ctx, hin, h->W, L.proj, n, h->proj, np, false, nullptr, 0, HyGlu{});
+    T* mixo = (T*)h->mixo + L.o0;
     int nsplit = 1;
     if (d.mixer == GL3_MIX_ATTENTION) {
         float* kc = h->slots + L.off_k;
         float* vc = h->slots + L.off_v;
-        const HyRot rot{d.rot_dims, L.rot_freq, d.v_unit_norm, d.v_rot ? L.vrot_freq : nullptr};
+        float* pk = d.pool > 0 ? h->slots + L.off_pk : nullptr;
+        float* pv = d.pool > 0 ? h->slots + L.off_pv : nullptr;
+        const HyRot rot{d.rot_dims, L.rot_freq, d.v_unit_norm, d.v_rot ? L.vrot_freq : nullptr, d.rot_interleaved};
+        const HyPrepX px{d.qk_bias ? L.pbias : nullptr, L.qn, L.kn, h->rowr};
+        if (d.qk_unit_norm == 2)
+            hipLaunchKernelGGL(hy_rowrms_kernel, dim3(n, 2), dim3(256), 0, st, h->proj, np, L.q_off, d.heads * d.dim, L.k_off, d.kv_heads * d.dim, px.bias, eps, h->rowr);
         hipLaunchKernelGGL(hy_attn_prep_kernel, dim3(n, d.heads + 2 * d.kv_heads), dim3(64), 0, st, h->proj, np, L.q_off, L.k_off, L.v_off, d.heads, d.kv_heads, d.dim,
-                           d.vdim, d.qk_unit_norm, eps, kc, vc, h->slot_floats, h->dyn, rot);
-        int32_t r = hy_attention(ctx, h->proj + L.q_off, np, kc, vc, d.heads, d.kv_heads, d.dim, d.vdim, d.scale, d.slope_log2, n, pos0, &nsplit, true, d.window, d.keep_first);
+                           d.vdim, d.qk_unit_norm, eps, kc, vc, h->slot_floats, h->dyn, rot, px);
+        if (d.pool > 0) {
+            const int done = (pos0 + n) / d.pool - pos0 / d.pool;          // blocks whose last position lies in this portion
+            if (done > 0)
+                hipLaunchKernelGGL(hy_pool_kernel, dim3(done, 2), dim3(256), 0, st, kc, vc, pk, pv, d.kv_heads * d.dim, d.kv_heads * d.vdim, d.pool, h->slot_floats, h->dyn, n);
+        }
+        int32_t r = hy_attention(ctx, h->proj + L.q_off, np, kc, vc, d.heads, d.kv_heads, d.dim, d.vdim, d.scale, d.slope_log2, n, pos0, &nsplit, true, d.window, d.keep_first,
+                                 pk, pv, d.pool);
         if (r != GL3_OK) return r;
         hipLaunchKernelGGL((hy_attn_merge_kernel<T>), dim3(n, d.heads), dim3(64), 0, st, h->part_acc, h->part_ml, d.heads, d.vdim, nsplit, d.softmax_sink,
-                           d.out_gate ? h->proj + L.g_off : nullptr, np, d.out_gate, mixo, d.heads * d.vdim, d.v_rot ? L.vrot_freq : nullptr, h->dyn);
+                           d.out_gate ? h->proj + L.g_off : nullptr, np, d.out_gate, mixo, ldo, d.v_rot ? L.vrot_freq : nullptr, h->dyn,
+                           d.softmax_sink == 2 ? L.sink : nullptr, L.out_mul);
+    } else if (d.mixer == GL3_MIX_MEMORY) {
+        const bool eg = d.mem_gates == GL3_MEM_EXP_GATES;
+        const int P = d.vdim + (eg ? 1 : 0), ldy = d.heads * P;
+        float *ga = h->gates, *gb = ga + (size_t)h->mb * h->max_heads, *ge = gb + (size_t)h->mb * h->max_heads;
+        if (eg)
+            hipLaunchKernelGGL(hy_mem_gates_kernel, dim3(d.heads), dim3(256), 0, st, h->proj, np, L.i_off, L.f_off, L.pbias, d.mem_gate_cap, d.heads, h->slots + L.off_m,
+                               h->slot_floats, h->dyn, n, ga, gb, ge);
+        HyScanArgs a{};
+        a.ksrc = h->proj; a.ldk = np; a.k_off = L.k_off; a.k_hstride = d.dim;
+        a.qsrc = h->proj; a.ldq = np; a.q_off = L.q_off; a.q_hstride = d.dim;
+        a.xsrc = h->proj; a.ldx = np; a.x_off = L.v_off;
+        a.k_mul = d.mem_k_mul != 0.f ? d.mem_k_mul : 1.f; a.q_mul = d.mem_q_mul != 0.f ? d.mem_q_mul : 1.f;
+        a.rot = HyScanRot{d.rot_dims, L.rot_freq, d.rot_interleaved};
+        a.mode = eg ? 1 : 2; a.ga = ga; a.gb = gb; a.decay = L.decay; a.ones_col = eg ? 1 : 0;
+        a.heads = d.heads; a.P = P; a.N = d.dim; a.G = d.heads;
+        a.state = h->slots + L.off_state; a.slot_stride = h->slot_floats; a.dyn = h->dyn; a.n = n; a.y = h->ssm_y; a.ldy = ldy;
+        hy_scan(ctx, a);
+        hipLaunchKernelGGL((hy_mem_out_kernel<T>), dim3(n, d.heads), dim3(64), 0, st, h->ssm_y, ldy, P, d.vdim, eg ? ge : nullptr, d.heads,
+                           d.mem_norm_weight ? L.ssm_norm : nullptr, h->proj, np, L.g_off, d.mem_gate_act, eps, L.out_mul, mixo, ldo);
     } else if (d.mixer == GL3_MIX_LATENT) {
         float* cc = h->slots + L.off_k;
         const int R = d.kv_rank;
@@ -639,7 +812,7 @@ static int32_t hy_mixer(gl3_ctx* ctx, HyLayer& L, int n, int pos0, int seq) {
             int32_t r = hy_attention(ctx, h->proj + L.q_off, np, h->kx, h->vx, d.heads, d.heads, d.dim, d.vdim, d.scale, 0.f, n, pos0, &nsplit, false);
             if (r != GL3_OK) return r;
             hipLaunchKernelGGL((hy_attn_merge_kernel<T>), dim3(n, d.heads), dim3(64), 0, st, h->part_acc, h->part_ml, d.heads, d.vdim, nsplit, d.softmax_sink,
-                               d.out_gate ? h->proj + L.g_off : nullptr, np, 1, mixo, d.heads * d.vdim, (const float*)nullptr, h->dyn);
+                               d.out_gate ? h->proj + L.g_off : nullptr, np, 1, mixo, ldo, (const float*)nullptr, h->dyn);
         } else {
             // A few tokens (decode): the query is carried into the latent's space and the attention core reads the latents themselves
             // (one shared key / value head, keys = values), then the weighted sum of latents is expanded.
@@ -655,10 +828,10 @@ static int32_t hy_mixer(gl3_ctx* ctx, HyLayer& L, int n, int pos0, int seq) {
                                (const float*)nullptr, 0, 0, h->oc, d.heads * R, (const float*)nullptr, h->dyn);
             if (n == 1)
                 hipLaunchKernelGGL((hy_headmm_kernel<T, 1>), dim3(1, d.heads, hy_cdiv(d.vdim, 64)), dim3(256), 0, st, h->oc, d.heads * R, R, d.vdim, L.wvT,
-                                   d.out_gate ? h->proj + L.g_off : nullptr, np, mixo, d.heads * d.vdim, n);
+                                   d.out_gate ? h->proj + L.g_off : nullptr, np, mixo, ldo, n);
             else
                 hipLaunchKernelGGL((hy_headmm_kernel<T, 8>), dim3(hy_cdiv(n, 8), d.heads, hy_cdiv(d.vdim, 64)), dim3(256), 0, st, h->oc, d.heads * R, R, d.vdim, L.wvT,
-                                   d.out_gate ? h->proj + L.g_off : nullptr, np, mixo, d.heads * d.vdim, n);
+                                   d.out_gate ? h->proj + L.g_off : nullptr, np, mixo, ldo, n);
         }
     } else {
         const int inner = d.heads * d.vdim, ch = hy_conv_ch(d), dt_off = 2 * inner + 2 * d.groups * d.state;
@@ -668,23 +841,31 @@ static int32_t hy_mixer(gl3_ctx* ctx, HyLayer& L, int n, int pos0, int seq) {
                            n, h->conv);
         if (d.conv > 1)
             hipLaunchKernelGGL(hy_conv_tail_kernel, dim3(hy_cdiv(ch, 256)), dim3(256), 0, st, h->proj, np, inner, ch, d.conv, tail, h->slot_floats, h->dyn, n);
-        // a column's states over NG lanes x NL registers: NL = 16 (32 for more than 1024 states, 8 / 4 for very small ones), NG a power of two
-        const int NL = d.state > 1024 ? 32 : d.state > 8 ? 16 : d.state > 4 ? 8 : 4;
-        int NG = 1;
-        while (NG * NL < d.state) NG *= 2;
-        const int cols = 4 * (64 / NG), Ns = NG * NL;
-        int TB = (int)(48 * 1024 / ((2 * (size_t)Ns + cols + 258) * 4));             // tokens staged per round: what fits 48 KB, at most 32
-        TB = std::max(1, std::min(32, TB));
-        const size_t smem = ((size_t)TB * (2 * Ns + cols + 256) + 2 * TB) * 4;
-        const dim3 grid(hy_cdiv(d.vdim, cols), d.heads);
-#define HY_SCAN(NLT)                                                                                                                                      \
-    hipLaunchKernelGGL((hy_ssm_scan_kernel<NLT>), grid, dim3(256), smem, st, h->proj, np, dt_off, h->conv, ch, d.heads, d.vdim, d.state, d.groups, NG, TB, L.dt_bias, \
-                       L.a_log, L.dskip, state, h->slot_floats, h->dyn, n, h->ssm_y)
-        if (NL == 4) HY_SCAN(4); else if (NL == 8) HY_SCAN(8); else if (NL == 16) HY_SCAN(16); else HY_SCAN(32);
-#undef HY_SCAN
-        hipLaunchKernelGGL((hy_gated_norm_kernel<T>), dim3(n, d.norm_groups), dim3(256), 0, st, h->ssm_y, h->proj, np, 0, inner, d.norm_groups, L.ssm_norm, eps, mixo);
+        HyScanArgs a{};
+        a.ksrc = h->conv; a.ldk = ch; a.k_off = inner; a.k_hstride = d.state;
+        a.qsrc = h->conv; a.ldq = ch; a.q_off = inner + d.groups * d.state; a.q_hstride = d.state;
+        a.xsrc = h->conv; a.ldx = ch; a.x_off = 0;
+        a.k_mul = a.q_mul = 1.f;
+        a.mode = 0; a.dtsrc = h->proj; a.ld_dt = np; a.dt_off = dt_off; a.dt_bias = L.dt_bias; a.A_log = L.a_log; a.Dp = L.dskip;
+        a.heads = d.heads; a.P = d.vdim; a.N = d.state; a.G = d.groups;
+        a.state = state; a.slot_stride = h->slot_floats; a.dyn = h->dyn; a.n = n; a.y = h->ssm_y; a.ldy = inner;
+        hy_scan(ctx, a);
+        hipLaunchKernelGGL((hy_gated_norm_kernel<T>), dim3(n, d.norm_groups), dim3(256), 0, st, h->ssm_y, h->proj, np, 0, inner, d.norm_groups, L.ssm_norm, eps, mixo, ldo);
     }
-    hy_gemm<T>(ctx, mixo, L.o.k, L.o, n, h->y, h->W, false, nullptr, 0, HyGlu{}, &h->y_parts);
+    return GL3_OK;
+}
+
+// The mixer sublayer of a layer on the n normed rows in h->h: one product for the inputs of every mixer of the layer, the mixers'
+// kernels, one product for their outputs (K-split parts in h->y, h->y_parts of them).
+template <typename T>
+static int32_t hy_mixer(gl3_ctx* ctx, HyLayer& L, int n, int pos0, int seq) {
+    gl3_hybrid_state* h = ctx->hy;
+    const int np = L.proj.rows;
+    hy_gemm<T>(ctx, (T*)h->h, h->W, L.proj, n, h->proj, np, false, nullptr, 0, HyGlu{});
+    int32_t r = hy_mixer_core<T>(ctx, L, np, L.mo_total, n, pos0, seq);
+    if (r == GL3_OK && L.side) r = hy_mixer_core<T>(ctx, *L.side, np, L.mo_total, n, pos0, seq);
+    if (r != GL3_OK) return r;
+    hy_gemm<T>(ctx, (T*)h->mixo, L.o.k, L.o, n, h->y, h->W, false, nullptr, 0, HyGlu{}, &h->y_parts);
     return GL3_OK;
 }
 
@@ -748,7 +929,7 @@ static void hy_moe(gl3_ctx* ctx, HyLayer& L, int n) {
     hy_gemm_grouped<T>(ctx, (const T*)h->eact, L.eff_pad, one_down, (size_t)W * L.edown.ld, P, max_tiles, few, h->eout, W, false, nullptr, 0, HyGlu{});
     if (d.shared_ff > 0) {
         T* act = (T*)h->mixo;
-        hy_gemm<T>(ctx, hb, W, L.gu, n, nullptr, 0, true, act, L.ff_pad, HyGlu{L.dense_limit, d.ff_alpha, d.ff_shift});
+        hy_gemm<T>(ctx, hb, W, L.gu, n, nullptr, 0, true, act, L.ff_pad, hy_ff_glu(L));
         hy_gemm<T>(ctx, act, L.ff_pad, L.down, n, h->y, W, false, nullptr, 0, HyGlu{}, &h->y_parts);
     }
 }
@@ -781,7 +962,7 @@ static int32_t hy_portion_plain(gl3_ctx* ctx, int seq, const int32_t* tokens, in
     hipLaunchKernelGGL((hy_embed_kernel<T>), dim3(n, n <= 32 ? hy_cdiv(W, 256) : 1), dim3(256), 0, st, h->tokens, (const T*)h->emb.w, h->X, W, 1, lstride, h->emb_scale, h->depth ? h->hist : nullptr);
     T* hb = (T*)h->h;
     HyResid base{};
-    base.x = h->X; base.W = W; base.eps = eps; base.ya_parts = 1;
+    base.x = h->X; base.W = W; base.eps = eps; base.ya_parts = 1; base.ya_mul = 1.f;
     {
         HyResid r = base;
         r.norm_w = h->L[0].norm1;
@@ -816,6 +997,22 @@ static int32_t hy_portion_plain(gl3_ctx* ctx, int seq, const int32_t* tokens, in
         if (rc != GL3_OK) return rc;
         HyResid r = base;
         r.ya = h->y; r.ya_parts = h->y_parts; r.ya_stride = (size_t)n * W;
+        if (h->parallel) {
+            // one norm, two readers: the feed-forward takes the same normed rows as the mixer, its down projection's parts follow the
+            // mixer's in y, and one residual update adds them all: x += residual multiplier * (mixer + feed-forward)
+            if (L.d.ff > 0) {
+                T* act = (T*)h->mixo;
+                int p2 = 1;
+                hy_gemm<T>(ctx, hb, W, L.gu, n, nullptr, 0, true, act, L.ff_pad, hy_ff_glu(L));
+                hy_gemm<T>(ctx, act, L.ff_pad, L.down, n, h->y + (size_t)h->y_parts * n * W, W, false, nullptr, 0, HyGlu{}, &p2);
+                r.ya_parts += p2;
+            }
+            r.ya_mul = h->resid_mul;
+            if (h->taps) r.tap = h->taps + (size_t)l * lstride;
+            if (!last) r.norm_w = h->L[l + 1].norm1;
+            hy_resid<T>(ctx, n, r, (T*)nullptr, hb);
+            continue;
+        }
         if (L.d.ff > 0) {
             r.norm_w = L.norm2;
             hy_resid<T>(ctx, n, r, (T*)nullptr, hb);
@@ -826,7 +1023,7 @@ static int32_t hy_portion_plain(gl3_ctx* ctx, int seq, const int32_t* tokens, in
                 if (L.d.shared_ff > 0) { r.ya = h->y; r.ya_parts = h->y_parts; r.ya_stride = (size_t)n * W; r.gate_z = h->sgz; r.gate_ld = 1; }
             } else {
                 T* act = (T*)h->mixo;
-                hy_gemm<T>(ctx, hb, W, L.gu, n, nullptr, 0, true, act, L.ff_pad, HyGlu{L.dense_limit, L.d.ff_alpha, L.d.ff_shift});
+                hy_gemm<T>(ctx, hb, W, L.gu, n, nullptr, 0, true, act, L.ff_pad, hy_ff_glu(L));
                 hy_gemm<T>(ctx, act, L.ff_pad, L.down, n, h->y, W, false, nullptr, 0, HyGlu{}, &h->y_parts);
                 r.ya = h->y; r.ya_parts = h->y_parts; r.ya_stride = (size_t)n * W;
             }
@@ -873,7 +1070,7 @@ static int32_t hy_portion(gl3_ctx* ctx, int seq, const int32_t* tokens, int n, i
         }
         if (ff) {
             T* act = (T*)h->mixo;
-            hy_gemm<T>(ctx, hb, W, L.gu, n, nullptr, 0, true, act, L.ff_pad, HyGlu{L.dense_limit, L.d.ff_alpha, L.d.ff_shift});
+            hy_gemm<T>(ctx, hb, W, L.gu, n, nullptr, 0, true, act, L.ff_pad, hy_ff_glu(L));
             hy_gemm<T>(ctx, act, L.ff_pad, L.down, n, h->y, W, false, nullptr, 0, HyGlu{}, &h->y_parts);
             const float* nin = last ? nullptr : h->L[l + 1].hc[0][0];
             const float* nw_ = last ? nullptr : h->L[l + 1].norm1;

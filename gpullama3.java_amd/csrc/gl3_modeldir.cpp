@@ -6,10 +6,12 @@
 #include <sys/stat.h>
 #include <unistd.h>
 
+#include <algorithm>
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <deque>
 #include <map>
 #include <memory>
 #include <string>
@@ -154,9 +156,11 @@ bool get_float(const JVal& o, const char* key, float& out, std::string& err) {
 }
 
 // ---- registered designs -----------------------------------------------------------------------------------------------------------
+// what a description points to besides the layer list (second mixers, decay lists): lives until gl3_create has copied it
+struct DescStore { std::deque<gl3_layer_desc> descs; std::deque<std::vector<float>> floats; };
 struct Design {
     const char* architecture;                                  // config.json "architecture"
-    bool (*describe)(const JVal& cfg, gl3_model_desc& d, std::vector<gl3_layer_desc>& layers, std::string& err);
+    bool (*describe)(const JVal& cfg, gl3_model_desc& d, std::vector<gl3_layer_desc>& layers, DescStore& store, std::string& err);
     // false: not a tensor of this design.  expert >= 0: the tensor is one expert's part of the stacked tensor `id` ([experts][..]); the
     // loader puts the parts together and uploads the whole once all of them are there
     bool (*tensor)(const std::string& name, int32_t& id, int32_t& layer, int32_t& expert);
@@ -165,7 +169,7 @@ struct Design {
 // Noditar: a list of layers of three mixer types behind hyper-connected residual streams.  The design fixes: unit-RMS q and k, distance
 // slopes 2^(-8 (h + 1) / H), one extra unit in the attention softmax's denominator (not in the latent attention's), sigmoid output
 // gates, and the feed-forward activation g sigmoid(1.702 g) (u + 1).
-bool noditar_describe(const JVal& cfg, gl3_model_desc& d, std::vector<gl3_layer_desc>& layers, std::string& err) {
+bool noditar_describe(const JVal& cfg, gl3_model_desc& d, std::vector<gl3_layer_desc>& layers, DescStore&, std::string& err) {
     d.arch = GL3_ARCH_NODITAR;
     d.weight_type = GL3_TYPE_BF16;
     if (!get_int(cfg, "vocab", d.vocab, err) || !get_int(cfg, "width", d.dim, err)) return false;
@@ -244,7 +248,7 @@ bool noditar_tensor(const std::string& name, int32_t& id, int32_t& layer, int32_
 // design fixes: norm weights kept as their deviation from one (weight = 1 + stored value), unit-RMS values, values rotated by their position and outputs
 // turned back, one sigmoid output gate per head, sigmoid router scores that scale the chosen experts' inputs, the expert activation
 // g sigmoid(1.702 g) (u + 1), a gated shared expert, a per-layer token input and the weighted average over all earlier layers' results.
-bool vonulix_describe(const JVal& cfg, gl3_model_desc& d, std::vector<gl3_layer_desc>& layers, std::string& err) {
+bool vonulix_describe(const JVal& cfg, gl3_model_desc& d, std::vector<gl3_layer_desc>& layers, DescStore&, std::string& err) {
     d.arch = GL3_ARCH_LAYERLIST;
     d.weight_type = GL3_TYPE_BF16;
     if (!get_int(cfg, "vocab", d.vocab, err) || !get_int(cfg, "width", d.dim, err)) return false;
@@ -328,7 +332,135 @@ bool vonulix_tensor(const std::string& name, int32_t& id, int32_t& layer, int32_
     return false;
 }
 
-const Design DESIGNS[] = {{"Noditar", noditar_describe, noditar_tensor}, {"Vonulix", vonulix_describe, vonulix_tensor}};
+// Kosusun: every layer is a parallel block — one RMS norm, whose output feeds the mixer and the feed-forward alike, and
+// x <- x + residual_mult (mixer + feed-forward).  Two layer types.  "parallel": two mixers side by side, `left` = grouped-query attention
+// (biased q / k / v, RMS norm with weights over the whole q and the whole k projection, interleaved rotary pairs with linear position
+// scaling, a sliding window plus the means of the blocks of `mask.pool` positions that lie wholly before it, a learned sink logit per
+// head) and `right` = retention (a matrix memory with a fixed decay per head, half-split rotary pairs, keys times dim^(-1/2), unit-RMS
+// heads times silu(W_g h)), added as left_scale * left + right_scale * right.  "mlstm": a matrix memory with exponential gates
+// (capped log gates, running maximum, normaliser; queries times dim^(-1/2); unit-RMS heads with a weight, times sigmoid(W_g h)).  The
+// feed-forward is gelu_tanh(W_gate h) * (W_up h) through W_down.  config.json gives every size and the constants named above; the
+// rest (the forms of the norms, gates and activations) is the design's and is fixed here.
+bool get_rot(const JVal& mx, gl3_layer_desc& ld, std::string& err) {
+    const JVal* rot = mx.get("rot");
+    if (!rot || rot->is_null()) return true;                 // no rotary positions
+    if (rot->kind != JVal::OBJ || !get_int(*rot, "dims", ld.rot_dims, err) || !get_float(*rot, "base", ld.rot_base, err)) {
+        if (err.empty()) err = "config: rot needs dims and base";
+        return false;
+    }
+    ld.rot_divide = 1.f;
+    if (const JVal* sc = rot->get("scaling"))
+        if (sc->kind == JVal::OBJ && !get_float(*sc, "factor", ld.rot_divide, err)) return false;
+    return true;
+}
+bool kosusun_attention(const JVal& mx, gl3_layer_desc& ld, std::string& err) {
+    ld.mixer = GL3_MIX_ATTENTION;
+    if (!get_int(mx, "heads", ld.heads, err) || !get_int(mx, "kv_heads", ld.kv_heads, err) || !get_int(mx, "dim", ld.dim, err) || !get_int(mx, "vdim", ld.vdim, err) ||
+        !get_float(mx, "scale", ld.scale, err) || !get_rot(mx, ld, err))
+        return false;
+    ld.qk_bias = 1; ld.qk_unit_norm = 2; ld.rot_interleaved = 1; ld.softmax_sink = 2;
+    if (const JVal* mask = mx.get("mask"))
+        if (mask->kind == JVal::OBJ) {
+            if (!get_int(*mask, "size", ld.window, err)) return false;
+            if (mask->get("pool") && !get_int(*mask, "pool", ld.pool, err)) return false;
+        }
+    return true;
+}
+bool kosusun_retention(const JVal& mx, gl3_layer_desc& ld, DescStore& store, std::string& err) {
+    ld.mixer = GL3_MIX_MEMORY;
+    ld.mem_gates = GL3_MEM_DECAY;
+    if (!get_int(mx, "heads", ld.heads, err) || !get_int(mx, "dim", ld.dim, err) || !get_int(mx, "vdim", ld.vdim, err) || !get_rot(mx, ld, err)) return false;
+    ld.kv_heads = ld.heads;
+    const JVal* dec = mx.get("decay");
+    if (!dec || dec->kind != JVal::ARR || (int)dec->arr.size() != ld.heads) { err = "config: retention needs a decay per head"; return false; }
+    store.floats.emplace_back();
+    for (const JVal& v : dec->arr) {
+        if (v.kind != JVal::NUM) { err = "config: decay must be numbers"; return false; }
+        store.floats.back().push_back((float)v.num);
+    }
+    ld.mem_decay = store.floats.back().data();
+    ld.mem_k_mul = (float)(1.0 / std::sqrt((double)std::max(1, ld.dim)));
+    ld.mem_gate_act = 0; ld.mem_norm_weight = 0;
+    return true;
+}
+bool kosusun_describe(const JVal& cfg, gl3_model_desc& d, std::vector<gl3_layer_desc>& layers, DescStore& store, std::string& err) {
+    d.arch = GL3_ARCH_LAYERLIST;
+    d.weight_type = GL3_TYPE_BF16;
+    if (!get_int(cfg, "vocab", d.vocab, err) || !get_int(cfg, "width", d.dim, err)) return false;
+    d.streams = 0;
+    d.parallel_block = 1;
+    d.embedding_scale = d.residual_scale = d.logit_scale = 1.f;
+    if (const JVal* e = cfg.get("embedding"))
+        if (e->kind == JVal::OBJ && e->get("scale") && !get_float(*e, "scale", d.embedding_scale, err)) return false;
+    if (cfg.get("residual_mult") && !get_float(cfg, "residual_mult", d.residual_scale, err)) return false;
+    if (cfg.get("logit_scale") && !get_float(cfg, "logit_scale", d.logit_scale, err)) return false;
+    const JVal* norm = cfg.get("norm");
+    if (!norm || !get_float(*norm, "eps", d.rms_eps, err)) { if (err.empty()) err = "config: missing norm.eps"; return false; }
+    const JVal* ls = cfg.get("layers");
+    if (!ls || ls->kind != JVal::ARR || ls->arr.empty()) { err = "config: 'layers' must be a non-empty list"; return false; }
+    for (const JVal& l : ls->arr) {
+        gl3_layer_desc ld{};
+        const JVal *ty = l.get("type"), *mx = l.get("mixer"), *mlp = l.get("mlp");
+        if (!ty || ty->kind != JVal::STR || !mx || mx->kind != JVal::OBJ) { err = "config: a layer needs 'type' and 'mixer'"; return false; }
+        if (ty->str == "parallel") {
+            const JVal *left = mx->get("left"), *right = mx->get("right");
+            if (!left || left->kind != JVal::OBJ || !right || right->kind != JVal::OBJ) { err = "config: a parallel mixer needs 'left' and 'right'"; return false; }
+            gl3_layer_desc rd{};
+            if (!kosusun_attention(*left, ld, err) || !kosusun_retention(*right, rd, store, err)) return false;
+            ld.out_scale = rd.out_scale = 1.f;
+            if (mx->get("left_scale") && !get_float(*mx, "left_scale", ld.out_scale, err)) return false;
+            if (mx->get("right_scale") && !get_float(*mx, "right_scale", rd.out_scale, err)) return false;
+            if (ld.out_scale == 0.f || rd.out_scale == 0.f) { err = "config: left_scale and right_scale must not be zero"; return false; }
+            store.descs.push_back(rd);
+            ld.beside = &store.descs.back();
+        } else if (ty->str == "mlstm") {
+            ld.mixer = GL3_MIX_MEMORY;
+            ld.mem_gates = GL3_MEM_EXP_GATES;
+            if (!get_int(*mx, "heads", ld.heads, err) || !get_int(*mx, "dim", ld.dim, err) || !get_int(*mx, "vdim", ld.vdim, err) ||
+                !get_float(*mx, "gate_cap", ld.mem_gate_cap, err))
+                return false;
+            ld.kv_heads = ld.heads;
+            ld.mem_q_mul = (float)(1.0 / std::sqrt((double)std::max(1, ld.dim)));
+            ld.mem_gate_act = 1; ld.mem_norm_weight = 1;
+        } else { err = "config: unknown layer type '" + ty->str + "'"; return false; }
+        if (mlp && !mlp->is_null()) {
+            const JVal* kind = mlp->get("kind");
+            if (!kind || kind->kind != JVal::STR || kind->str != "dense") { err = "config: mlp.kind must be 'dense'"; return false; }
+            if (!get_int(*mlp, "ff", ld.ff, err)) return false;
+            ld.ff_act = 1;
+        }
+        layers.push_back(ld);
+    }
+    d.n_layers = (int32_t)layers.size();
+    return true;
+}
+
+bool kosusun_tensor(const std::string& name, int32_t& id, int32_t& layer, int32_t& expert) {
+    static const std::map<std::string, int> global = {{"embed", GL3_T_TOKEN_EMBD}, {"head", GL3_T_OUTPUT}, {"final.norm", GL3_T_OUTPUT_NORM}};
+    static const std::map<std::string, int> leaf = {{"norm1", GL3_T_ATTN_NORM}, {"mlp.gate", GL3_T_W1}, {"mlp.up", GL3_T_W3}, {"mlp.down", GL3_T_W2}};
+    // tensors of one mixer, after "mix." (mlstm), "mix.left." (attention) or "mix.right." (retention)
+    static const std::map<std::string, int> mix = {
+        {"q", GL3_T_WQ}, {"k", GL3_T_WK}, {"v", GL3_T_WV}, {"o", GL3_T_WO}, {"g", GL3_T_ATTN_GATE}, {"q.b", GL3_T_BQ}, {"k.b", GL3_T_BK}, {"v.b", GL3_T_BV},
+        {"q.norm", GL3_T_ATTN_Q_NORM}, {"k.norm", GL3_T_ATTN_K_NORM}, {"sink", GL3_T_ATTN_SINK}, {"norm", GL3_T_SSM_NORM}, {"i", GL3_T_MEM_IGATE},
+        {"f", GL3_T_MEM_FGATE}, {"i.b", GL3_T_MEM_IGATE_BIAS}, {"f.b", GL3_T_MEM_FGATE_BIAS}};
+    expert = -1;
+    auto g = global.find(name);
+    if (g != global.end()) { id = g->second; layer = 0; return true; }
+    std::string lf;
+    if (!split_layer_name(name, layer, lf)) return false;
+    auto f = leaf.find(lf);
+    if (f != leaf.end()) { id = f->second; return true; }
+    if (lf.compare(0, 4, "mix.") != 0) return false;
+    std::string rest = lf.substr(4);
+    if (rest.compare(0, 5, "left.") == 0) rest = rest.substr(5);
+    else if (rest.compare(0, 6, "right.") == 0) { rest = rest.substr(6); layer |= GL3_LAYER_BESIDE; }
+    auto m = mix.find(rest);
+    if (m == mix.end()) return false;
+    id = m->second;
+    return true;
+}
+
+const Design DESIGNS[] = {{"Noditar", noditar_describe, noditar_tensor}, {"Vonulix", vonulix_describe, vonulix_tensor}, {"Kosusun", kosusun_describe, kosusun_tensor}};
 
 struct Mapping {
     void* p = MAP_FAILED; size_t n = 0;
@@ -368,8 +500,9 @@ static int32_t load_model_dir(const char* dir, const gl3_model_desc* opts, gl3_c
     gl3_model_desc d{};
     d.struct_size = sizeof d;
     std::vector<gl3_layer_desc> layers;
+    DescStore store;
     std::string err;
-    if (!design->describe(cfg, d, layers, err)) { g_dir_err = err; return GL3_E_ARG; }
+    if (!design->describe(cfg, d, layers, store, err)) { g_dir_err = err; return GL3_E_ARG; }
     d.layer_descs = layers.data();
     d.ctx = opts && opts->ctx > 0 ? opts->ctx : 4096;
     d.max_batch = opts && opts->max_batch > 0 ? opts->max_batch : 512;
@@ -427,7 +560,7 @@ static int32_t load_model_dir(const char* dir, const gl3_model_desc* opts, gl3_c
     }
     for (auto& st : stacks) {
         const int32_t layer = st.first.first, id = st.first.second;
-        const int want = layer >= 0 && layer < (int)layers.size() ? layers[layer].experts : 0;
+        const int want = layer >= 0 && layer < (int)layers.size() ? layers[layer].experts : 0;          // (a second mixer has no experts)
         const Part& first = st.second.begin()->second;
         bool ok = (int)st.second.size() == want && st.second.rbegin()->first == want - 1;
         for (auto& pt : st.second) ok = ok && pt.second.n == first.n && pt.second.type == first.type;

@@ -21,7 +21,9 @@ FLAG_VECTOR_512, FLAG_VECTOR_128 = 32, 64      # -Dllama.VectorBitSize (default 
 FLAG_F32_COMPUTE = 128                         # layer-list family: float32 matrices and products
 ARCH_NODITAR = ARCH_LAYERLIST = 6      # the layer-list family; its designs differ in parameters only
 TYPE_F32, TYPE_BF16 = 0, 30
-MIX_ATTENTION, MIX_LATENT, MIX_SSM = 0, 1, 2
+MIX_ATTENTION, MIX_LATENT, MIX_SSM, MIX_MEMORY = 0, 1, 2, 3
+MEM_DECAY, MEM_EXP_GATES = 0, 1
+LAYER_BESIDE = 1 << 30
 K_NAMES = ["matvec_qkv", "matvec_wo", "matvec_gateup", "matvec_down", "matvec_logits", "attention", "other", "collective"]
 
 T_IDS = {"token_embd.weight": 0, "output_norm.weight": 1, "output.weight": 2, "attn_norm.weight": 3,
@@ -55,7 +57,11 @@ class LayerDesc(C.Structure):
                 ("qk_unit_norm", C.c_int32), ("slope_log2", C.c_float), ("softmax_sink", C.c_int32), ("out_gate", C.c_int32),
                 ("rot_dims", C.c_int32), ("rot_base", C.c_float), ("rot_divide", C.c_float), ("v_unit_norm", C.c_int32),
                 ("v_rot", C.c_int32), ("window", C.c_int32), ("keep_first", C.c_int32), ("experts", C.c_int32), ("top", C.c_int32),
-                ("shared_ff", C.c_int32), ("shared_limit", C.c_float)]
+                ("shared_ff", C.c_int32), ("shared_limit", C.c_float), ("ff_act", C.c_int32),
+                ("qk_bias", C.c_int32), ("rot_interleaved", C.c_int32), ("pool", C.c_int32),
+                ("mem_gates", C.c_int32), ("mem_decay", C.POINTER(C.c_float)), ("mem_q_mul", C.c_float), ("mem_k_mul", C.c_float),
+                ("mem_gate_cap", C.c_float), ("mem_norm_weight", C.c_int32), ("mem_gate_act", C.c_int32),
+                ("beside", C.c_void_p), ("out_scale", C.c_float)]          # beside: address of another LayerDesc
 
 
 class ModelDesc(C.Structure):
@@ -67,7 +73,7 @@ class ModelDesc(C.Structure):
                 ("residual_scale", C.c_float), ("logit_scale", C.c_float),
                 ("n_experts", C.c_int32), ("n_experts_used", C.c_int32), ("moe_hidden", C.c_int32),
                 ("streams", C.c_int32), ("layer_descs", C.POINTER(LayerDesc)),
-                ("norm_offset", C.c_float), ("side_dim", C.c_int32), ("depth_mix", C.c_int32)]
+                ("norm_offset", C.c_float), ("side_dim", C.c_int32), ("depth_mix", C.c_int32), ("parallel_block", C.c_int32)]
 
 
 class KernelTimes(C.Structure):

@@ -71,19 +71,30 @@ enum { GL3_ARCH_LLAMA = 0, GL3_ARCH_QWEN3 = 1, GL3_ARCH_QWEN2 = 2,
                               * gl3_layer_desc; several residual streams mixed by per-sublayer tables, or one plain residual with an optional
                               * weighted average over all earlier layers' results; bfloat16 or float32 matrices
                               * (GL3_TYPE_BF16, GL3_FLAG_F32_COMPUTE); model folders with config.json + model.safetensors (gl3_load_model_dir) */
-       GL3_ARCH_LAYERLIST = 6 /* the same family under its own name: the registered designs (Noditar, Vonulix) differ only in the
-                              * parameters of gl3_model_desc / gl3_layer_desc that their `describe` fills in */ };
+       GL3_ARCH_LAYERLIST = 6 /* the same family under its own name: the registered designs (Noditar, Vonulix, Kosusun) differ only in
+                              * the parameters of gl3_model_desc / gl3_layer_desc that their `describe` fills in */ };
 
 /* token mixers of a layer-list model (gl3_layer_desc.mixer) */
 enum { GL3_MIX_ATTENTION = 0,   /* grouped-query softmax attention over cached keys / values; optional unit-RMS q and k, linear distance
                                  * penalty per head, extra unit in the softmax denominator, sigmoid output gate (per element or per head),
                                  * rotary positions on part of q / k, unit-RMS and rotated values, sliding window with kept first keys */
        GL3_MIX_LATENT = 1,      /* attention whose keys and values are expanded from one cached low-rank latent per token */
-       GL3_MIX_SSM = 2 };       /* selective state-space recurrence (scalar decay per head) behind a short causal convolution */
+       GL3_MIX_SSM = 2,         /* selective state-space recurrence (scalar decay per head) behind a short causal convolution */
+       GL3_MIX_MEMORY = 3 };    /* matrix memory per head, S_t = a_t S_(t-1) + b_t k_t v_t^T, o_t = S_t^T q_t, float32 state carried per sequence:
+                                 * a fixed decay per head (retention) or exponential gates with a running maximum and a normaliser (mLSTM) */
+
+/* gl3_layer_desc.mem_gates: how a matrix memory gets a_t and b_t */
+enum { GL3_MEM_DECAY = 0,       /* a = mem_decay[head], b = 1; no normaliser: o = S^T q */
+       GL3_MEM_EXP_GATES = 1 }; /* log gates from two projections with biases: i = cap tanh(z_i / cap), f = logsigmoid(cap tanh(z_f / cap));
+                                 * m_t = max(f + m_(t-1), i), m_0 = 0; a = e^(f + m_(t-1) - m_t), b = e^(i - m_t); n_t = a n + b k;
+                                 * o = S^T q / (max(|n . q|, e^(-m_t)) + 1e-6) */
+
+/* gl3_upload_tensor: `layer` + GL3_LAYER_BESIDE addresses the second mixer of a layer (gl3_layer_desc.beside) */
+#define GL3_LAYER_BESIDE (1 << 30)
 
 /* One layer of a layer-list model: the mixer, its sizes, the feed-forward behind it, and the constants of each mechanism (a design
  * fixes them; another design that shares the mechanism passes its own). */
-typedef struct {
+typedef struct gl3_layer_desc {
     int32_t mixer;              /* GL3_MIX_* */
     int32_t heads, kv_heads;    /* query heads; key / value heads (attention), = heads otherwise */
     int32_t dim, vdim;          /* per-head query / key size and value size (ssm: vdim = head width) */
@@ -114,6 +125,30 @@ typedef struct {
     int32_t experts, top;
     int32_t shared_ff;
     float   shared_limit;
+    int32_t ff_act;             /* 0: act = g sigmoid(ff_alpha g) (u + ff_shift); 1: act = gelu_tanh(g) u */
+    /* attention, further switches (each usable alone).  qk_bias: q, k and v projections have biases (GL3_T_BQ / BK / BV).
+     * qk_unit_norm = 2: RMS norm over the WHOLE q projection (all heads at once) and the whole k projection, with plain weights
+     * GL3_T_ATTN_Q_NORM [heads dim] / GL3_T_ATTN_K_NORM [kv_heads dim], after the bias and before the rotation.  rot_interleaved:
+     * rotary pairs are entries (2 i, 2 i + 1) instead of (i, i + rot_dims / 2) (also read by a matrix memory).  softmax_sink = 2: a
+     * learned logit per head (GL3_T_ATTN_SINK [heads]) joins the denominator as e^sink, unscaled, without key or value.
+     * pool > 0 (needs window > 0): beside the window's keys, query i sees one key / value per block of `pool` positions that lies
+     * wholly before its window (block b = positions b pool .. b pool + pool - 1, seen if b pool + pool - 1 <= i - window): the means of
+     * the block's cached keys and values; positions between the seen blocks and the window are not seen at all */
+    int32_t qk_bias, rot_interleaved, pool;
+    /* matrix memory (GL3_MIX_MEMORY): heads, dim (keys / queries), vdim; rot_* turn q and k as in attention; q and k are multiplied by
+     * mem_q_mul / mem_k_mul (0 = 1) after the rotation.  The head's output is divided by its root mean square, multiplied by the weight
+     * GL3_T_SSM_NORM [heads vdim] if mem_norm_weight, and by act(W_g h) (GL3_T_ATTN_GATE, act = silu for mem_gate_act 0, sigmoid for 1).
+     * mem_decay: heads values (copied by gl3_create).  GL3_MEM_EXP_GATES: gate projections GL3_T_MEM_IGATE / FGATE [heads x width] and
+     * their biases GL3_T_MEM_IGATE_BIAS / FGATE_BIAS [heads], cap = mem_gate_cap */
+    int32_t mem_gates;
+    const float* mem_decay;
+    float   mem_q_mul, mem_k_mul, mem_gate_cap;
+    int32_t mem_norm_weight, mem_gate_act;
+    /* Two mixers side by side: `beside` (copied by gl3_create; its own beside, ff and experts are ignored) reads the same normed input
+     * and the layer's mixer output is out_scale * this + beside->out_scale * that (out_scale 0 = 1), each through its own output
+     * projection.  Its tensors are uploaded with layer + GL3_LAYER_BESIDE. */
+    const struct gl3_layer_desc* beside;
+    float   out_scale;
 } gl3_layer_desc;
 
 /* ggml tensor types of the wire format (J/tensor/GGMLType.java:5-21) */
@@ -172,7 +207,12 @@ enum {
     GL3_T_SIDE_GATE = 44,          /*                                                [side_dim x width]                  */
     GL3_T_SIDE_PROJ = 45,          /*                                                [width x side_dim]                  */
     GL3_T_SIDE_NORM = 46,          /* plain weight of the unit-RMS norm behind the projection  [width]                   */
-    GL3_T_COUNT = 47
+    GL3_T_ATTN_SINK = 47,          /* attention: learned logit per head in the softmax denominator  [heads]              */
+    GL3_T_MEM_IGATE = 48,          /* matrix memory: input gate projection           [heads x width]                     */
+    GL3_T_MEM_FGATE = 49,          /* matrix memory: forget gate projection          [heads x width]                     */
+    GL3_T_MEM_IGATE_BIAS = 50,     /*                                                [heads]                             */
+    GL3_T_MEM_FGATE_BIAS = 51,     /*                                                [heads]                             */
+    GL3_T_COUNT = 52
 };
 
 /* gl3_model_desc.flags */
@@ -240,6 +280,10 @@ typedef struct {
     float   norm_offset;
     int32_t side_dim;
     int32_t depth_mix;
+    /* layer-list family with streams == 0, parallel_block != 0: every layer has ONE norm and both sublayers read its output,
+     * x <- x + residual_scale (mixer(norm1 x) + ff(norm1 x)) (residual_scale, above, 0 = 1; no GL3_T_FFN_NORM).  logit_scale (above,
+     * 0 = 1) multiplies the family's logits. */
+    int32_t parallel_block;
 } gl3_model_desc;
 
 /* Per-kernel-class device time of one instrumented decode step (HIP events around every launch). */
