@@ -1,0 +1,468 @@
+"""The Kosusun design (layer-list family: parallel blocks, attention with pooled blocks behind a window beside retention, mLSTM layers)
+on the GPU against the plain float64 restatement in tests/kosusun_ref.py.
+
+Every test makes its own small configuration and random bfloat16-representable weights, writes them as a model folder and loads that
+through the product's loader.  float32 plans are held to 2e-4 (root mean square of the logit difference over the root mean square of
+the logits), bfloat16 plans to 6e-2.  Where random weights would hide a fault, queries are made multiples of keys on the entries that
+do not turn, so that a token attends to the earlier occurrences of the same token wherever they are, as single keys inside the window
+and as parts of pooled blocks before it: one key or one block more or less then moves the logits by far more than the bound, and the
+tests check that by moving the restatement's own window and block edge by one.
+"""
+import copy
+import json
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+import __graft_entry__ as ge
+import kosusun_ref as R
+
+pytestmark = pytest.mark.gpu
+F32_TOL, BF16_TOL = 2e-4, 6e-2
+
+
+@pytest.fixture(scope="module")
+def hy():
+    from importlib import import_module
+    ge.load_package()
+    return import_module(ge.PKG_NAME + ".hybrid")
+
+
+def attn(heads=4, kv_heads=2, dim=24, vdim=40, scale=0.3, size=37, pool=5, rot_dims=16, base=10000.0, factor=4.0):
+    rot = {"base": base, "dims": rot_dims}
+    if factor is not None:
+        rot["scaling"] = {"factor": factor}
+    mask = {"size": size}
+    if pool:
+        mask["pool"] = pool
+    return {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale, "mask": mask, "rot": rot}
+
+
+def ret(heads=3, dim=16, vdim=24, rot_dims=8, base=500.0, decay=None):
+    return {"heads": heads, "dim": dim, "vdim": vdim, "rot": {"base": base, "dims": rot_dims},
+            "decay": decay or [1.0 - 2.0 ** -(3 + i) for i in range(heads)]}
+
+
+def par(left=None, right=None, ff=56, ls=0.8, rs=1.3):
+    return {"type": "parallel", "mixer": {"left": left or attn(), "right": right or ret(), "left_scale": ls, "right_scale": rs},
+            "mlp": {"kind": "dense", "ff": ff} if ff else None}
+
+
+def mls(heads=3, dim=20, vdim=28, cap=12.0, ff=40):
+    return {"type": "mlstm", "mixer": {"heads": heads, "dim": dim, "vdim": vdim, "gate_cap": cap}, "mlp": {"kind": "dense", "ff": ff} if ff else None}
+
+
+def config(layers, width=88, vocab=131, emb_scale=2.5, eps=1e-5, mult=0.6, logit_scale=0.37):
+    return {"architecture": "Kosusun", "vocab": vocab, "width": width, "embedding": {"scale": emb_scale}, "norm": {"eps": eps}, "residual_mult": mult,
+            "logit_scale": logit_scale, "layers": layers}
+
+
+class Model:
+    def __init__(self, hy, tmp_path, cfg, seed, tweak=None, tied=False):
+        self.cfg, self.w = cfg, R.random_weights(cfg, seed, tied)
+        if tweak:
+            tweak(cfg, self.w)
+            self.w = {k: R.bf16_round(v) for k, v in self.w.items()}
+        self.dir = str(tmp_path / ("m%d" % seed))
+        hy.save_model_dir(self.dir, cfg, self.w)
+        self.w64 = R.to_f64(self.w)
+        self.hy = hy
+
+    def plan(self, dtype="float32", **kw):
+        return self.hy.HybridPlan.from_dir(self.dir, dtype=dtype, **kw)
+
+    def ref(self, tokens, cfg=None, **kw):
+        return R.forward(cfg or self.cfg, self.w64, tokens, **kw)
+
+    def tokens(self, n, seed=0, vocab=None):
+        toks = np.random.default_rng(1000 + seed).integers(0, vocab or self.cfg["vocab"], n).astype(np.int32)
+        return toks, self.ref(toks)
+
+
+def err(got, want):
+    d = got - want
+    d = d - d.mean(axis=-1, keepdims=True)
+    w = want - want.mean(axis=-1, keepdims=True)
+    return float(np.sqrt((d ** 2).mean(axis=-1)).max() / np.sqrt((w ** 2).mean()))
+
+
+def whole(plan, toks, want=None):
+    want = list(range(len(toks))) if want is None else want
+    s = plan.acquire()
+    out = plan.step(s, toks, 0, want)
+    plan.release(s)
+    return out
+
+
+def stepwise(plan, toks, sizes):
+    """The sequence in steps of the given sizes (the last size repeats), all logits."""
+    s = plan.acquire()
+    rows, p, i = [], 0, 0
+    while p < len(toks):
+        c = min(sizes[min(i, len(sizes) - 1)], len(toks) - p)
+        rows.append(plan.step(s, toks[p:p + c], p, list(range(c))))
+        p += c
+        i += 1
+    plan.release(s)
+    return np.concatenate(rows)
+
+
+# ---- each mechanism alone: one layer, the mechanism's sizes and constants varied ----------------------------------------------------------
+SINGLE = [
+    ("parallel_plain", par(), {}),
+    ("parallel_no_feed_forward", par(ff=0), {}),
+    ("mlstm_plain", mls(), {}),
+    ("mlstm_no_feed_forward", mls(ff=0), {}),
+    ("every_head_its_own_keys", par(left=attn(heads=3, kv_heads=3, dim=18, vdim=70)), {}),
+    ("one_kv_head", par(left=attn(heads=6, kv_heads=1, dim=32, vdim=16)), {}),
+    ("wide_heads", par(left=attn(heads=2, kv_heads=1, dim=200, vdim=300, rot_dims=64), right=ret(heads=1, dim=136, vdim=72, rot_dims=136), ff=0), {}),
+    ("rotary_all_dims_unscaled", par(left=attn(rot_dims=24, factor=None), right=ret(rot_dims=16)), {}),
+    ("rotary_two_dims", par(left=attn(rot_dims=2, factor=7.5, base=50.0), right=ret(rot_dims=2, base=3.0)), {}),
+    ("window_1_pool_1", par(left=attn(size=1, pool=1)), {}),
+    ("window_without_pool", par(left=attn(size=20, pool=0)), {}),
+    ("pool_wider_than_window", par(left=attn(size=3, pool=11)), {}),
+    ("window_larger_than_prompt", par(left=attn(size=500, pool=4)), {}),
+    ("window_and_pool_of_a_tile", par(left=attn(size=64, pool=64)), {"n": 200}),
+    ("pool_2_many_blocks", par(left=attn(size=7, pool=2)), {"n": 300}),
+    ("scales_of_one", par(ls=1.0, rs=1.0), {"mult": 1.0, "logit_scale": 1.0, "emb_scale": 1.0}),
+    ("retention_never_forgets", par(right=ret(heads=2, decay=[1.0, 0.5])), {}),
+    ("retention_small_and_odd", par(right=ret(heads=5, dim=6, vdim=7, rot_dims=4)), {}),
+    ("retention_one_state_row", par(right=ret(heads=2, dim=2, vdim=3, rot_dims=2)), {}),
+    ("mlstm_one_head_wide", mls(heads=1, dim=72, vdim=130), {}),
+    ("mlstm_many_small_heads", mls(heads=11, dim=4, vdim=6), {}),
+    ("mlstm_tight_gate_cap", mls(cap=0.75), {}),
+    ("widths_not_multiples_of_four", par(left=attn(heads=4, kv_heads=2, dim=18, vdim=22, rot_dims=6), right=ret(heads=3, dim=10, vdim=9, rot_dims=6), ff=33),
+     {"width": 75, "vocab": 53}),
+    ("mlstm_odd_widths", mls(heads=3, dim=9, vdim=11, ff=17), {"width": 50, "vocab": 77}),
+    ("twelve_heads_on_two", par(left=attn(heads=12, kv_heads=2, dim=8, vdim=12, rot_dims=8)), {"width": 80}),
+    ("wide_model", par(left=attn(heads=2, kv_heads=1, dim=32, vdim=32), right=ret(heads=2, dim=32, vdim=32), ff=96), {"width": 1024, "vocab": 64, "n": 40}),
+    ("wide_model_mlstm", mls(heads=2, dim=32, vdim=48, ff=2048), {"width": 1024, "vocab": 64, "n": 40}),
+]
+
+
+@pytest.mark.parametrize("name,lay,kw", SINGLE, ids=[s[0] for s in SINGLE])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_single_mechanism(hy, tmp_path, name, lay, kw, dtype):
+    kw = dict(kw)
+    n = kw.pop("n", 75)
+    m = Model(hy, tmp_path, config([lay], **kw), seed=len(name))
+    toks, ref = m.tokens(n)
+    plan = m.plan(dtype, ctx=max(128, n))
+    got = whole(plan, toks)
+    plan.close()
+    assert err(got, ref) < (F32_TOL if dtype == "float32" else BF16_TOL)
+
+
+def test_tied_head(hy, tmp_path):
+    m = Model(hy, tmp_path, config([mls(), par()]), seed=3, tied=True)
+    toks, ref = m.tokens(30)
+    plan = m.plan("float32", ctx=32)
+    assert err(whole(plan, toks), ref) < F32_TOL
+    plan.close()
+
+
+MIXED = [mls(heads=2, dim=24, vdim=16, ff=0), par(),
+         par(left=attn(heads=6, kv_heads=3, dim=16, vdim=32, scale=0.4, size=70, pool=9, rot_dims=8, base=500.0, factor=1.5), right=ret(heads=2, dim=40, vdim=12, rot_dims=40), ff=24),
+         mls(heads=4, dim=12, vdim=20, cap=5.0, ff=64), par(left=attn(heads=2, kv_heads=2, dim=40, vdim=24, size=9, pool=3, rot_dims=40, factor=None), ff=0)]
+
+
+def test_layer_taps(hy, tmp_path):
+    """The residual that leaves every layer against the restatement, layer by layer."""
+    m = Model(hy, tmp_path, config(MIXED, width=96), seed=41)
+    toks, ref = m.tokens(90)
+    plan = m.plan("float32", ctx=96, layer_taps=True)
+    taps = []
+    m.ref(toks, taps=taps)
+    got = whole(plan, toks)
+    for l, t in enumerate(taps):
+        rows = plan.layer_rows(l, len(toks))
+        assert np.abs(rows - t).max() < 1e-4 * max(1.0, np.abs(t).max()), l
+    plan.close()
+    assert err(got, ref) < F32_TOL
+
+
+# ---- prompts cut into portions, decoding token by token -----------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_prefill_equals_token_by_token_and_portions(hy, tmp_path, dtype):
+    m = Model(hy, tmp_path, config(MIXED), seed=7)
+    n = 150
+    toks, ref = m.tokens(n)
+    tol = F32_TOL if dtype == "float32" else BF16_TOL
+    plan = m.plan(dtype, ctx=160, max_batch=64)              # the whole prompt runs as portions of 64 inside one step, too
+    assert err(whole(plan, toks), ref) < tol
+    assert err(stepwise(plan, toks, [1]), ref) < tol
+    for sizes in ([2, 3, 2, 64, 5, 1, 1, 37, 2, 33], [70, 2, 2, 2, 74], [1, 149], [9, 2]):
+        assert err(stepwise(plan, toks, sizes), ref) < tol, sizes
+    plan.close()
+
+
+def test_logits_do_not_depend_on_the_cut(hy, tmp_path):
+    """float32: the same position through different cuts agrees to rounding."""
+    m = Model(hy, tmp_path, config(MIXED), seed=8)
+    toks, _ = m.tokens(90)
+    plan = m.plan("float32", ctx=128)
+    a = whole(plan, toks)
+    b = stepwise(plan, toks, [41, 2, 47])
+    c = stepwise(plan, toks, [1])
+    plan.close()
+    assert err(b, a) < 2e-5 and err(c, a) < 2e-5
+
+
+# ---- slots ---------------------------------------------------------------------------------------------------------------------------------
+def test_interleaved_requests_and_slot_reuse(hy, tmp_path):
+    """Unequal requests whose steps alternate give what each gives alone; a slot that a long request left (cache rows, pooled rows,
+    memory states, running maxima) is clean for the next."""
+    m = Model(hy, tmp_path, config(MIXED), seed=9)
+    (ta, ra), (tb, rb), (tc, rc) = m.tokens(60, 1), m.tokens(45, 2), m.tokens(30, 3)
+    plan = m.plan("float32", ctx=64, n_seqs=2)
+    a, b = plan.acquire(), plan.acquire()
+    assert a != b
+    with pytest.raises(hy.hip.Gl3Error):
+        plan.acquire()                                   # both slots are taken
+    ga, gb = [], []
+    ga.append(plan.step(a, ta[:20], 0, list(range(20))))
+    gb.append(plan.step(b, tb[:7], 0, list(range(7))))
+    ga.append(plan.step(a, ta[20:21], 20, [0]))
+    gb.append(plan.step(b, tb[7:40], 7, list(range(33))))
+    ga.append(plan.step(a, ta[21:], 21, list(range(39))))
+    for i in range(40, 45):
+        gb.append(plan.step(b, tb[i:i + 1], i, [0]))
+    assert err(np.concatenate(ga), ra) < F32_TOL and err(np.concatenate(gb), rb) < F32_TOL
+    plan.release(a)
+    c = plan.acquire()
+    assert c == a
+    gc = [plan.step(c, tc[:1], 0, [0]), plan.step(c, tc[1:3], 1, [0, 1]), plan.step(c, tc[3:], 3, list(range(27)))]
+    assert err(np.concatenate(gc), rc) < F32_TOL
+    with pytest.raises(hy.hip.Gl3Error):
+        plan.step(c, tc[:2], 7, [])                      # neither a continuation nor a restart
+    assert err(plan.step(b, tc, 0, list(range(30))), rc) < F32_TOL          # a restart at position 0 on a live slot starts clean as well
+    plan.close()
+
+
+def test_decode_batch_over_slots(hy, tmp_path):
+    m = Model(hy, tmp_path, config(MIXED[:3]), seed=10)
+    (ta, ra), (tb, rb) = m.tokens(12, 4), m.tokens(9, 5)
+    plan = m.plan("float32", ctx=32, n_seqs=2)
+    a, b = plan.acquire(), plan.acquire()
+    plan.step(a, ta[:11], 0, [])
+    plan.step(b, tb[:8], 0, [])
+    logits, ids = plan.forward_decode_batch([ta[11], tb[8]], [a, b], [11, 8])
+    plan.close()
+    assert err(logits, np.stack([ra[11], rb[8]])) < F32_TOL and list(ids) == list(np.argmax(logits, axis=1))
+
+
+# ---- windows, pooled blocks, far keys: a token looks for its own earlier occurrences ------------------------------------------------------
+def lookup_heads(cfg, w, copy_score=3.0):
+    """Attention: every query head becomes a multiple of its key head on the entries that do not turn, and zero on those that do
+    (weights, biases and norm weights alike): the score of a key depends on its token only, a token finds every earlier copy of itself
+    `copy_score` above the other keys, and a pooled block scores by the share of copies it holds.  The score is kept moderate: the mean
+    of a block's keys divides a copy's score by the block's length, and a block must still hold a visible share of the softmax.  The
+    embedding is made small and the retention's share too, so that what the attention gathers decides the logits.
+    Retention: queries become copies of keys as well, one head never forgets (decay 1): copies hundreds of positions back count."""
+    w["embed"] = w["embed"] * 0.05
+    for i, lay in enumerate(cfg["layers"]):
+        if lay["type"] != "parallel":
+            continue
+        mx = lay["mixer"]["left"]
+        H, G, D, rd = mx["heads"], mx["kv_heads"], mx["dim"], mx["rot"]["dims"]
+        pre = "l%d.mix.left." % i
+        k = w[pre + "k"].reshape(G, D, -1).copy()
+        kb = np.zeros((G, D), np.float32)
+        k[:, :rd] = 0.0
+        w[pre + "k"], w[pre + "k.b"] = k.reshape(G * D, -1), kb.reshape(G * D)
+        w[pre + "q"] = np.repeat(k, H // G, axis=0).reshape(H * D, -1).astype(np.float32)
+        w[pre + "q.b"] = np.zeros(H * D, np.float32)
+        w[pre + "k.norm"] = np.ones(G * D, np.float32)
+        # both projections leave their norm with a mean square of one over ALL entries: the D - rd live entries of a head carry D / (D - rd) each
+        w[pre + "q.norm"] = np.full(H * D, copy_score / mx["scale"] / D, np.float32)
+        w[pre + "sink"] = np.full(H, -4.0, np.float32)
+        lay["mixer"]["right_scale"] = 0.05
+        r = lay["mixer"]["right"]
+        pre = "l%d.mix.right." % i
+        kr = w[pre + "k"].reshape(r["heads"], r["dim"], -1).copy()
+        kr[:, :r["rot"]["dims"]] = 0.0
+        w[pre + "k"] = kr.reshape(r["heads"] * r["dim"], -1)
+        w[pre + "q"] = w[pre + "k"].copy()
+        r["decay"] = [1.0] + list(r["decay"][1:])
+
+
+EDGE_CASES = [(37, 5, 150, 120), (64, 8, 200, 190), (65, 64, 330, 300), (63, 1, 129, 60), (128, 20, 400, 380), (40, 7, 530, 505)]
+
+
+@pytest.mark.parametrize("size,pool,n,decode_from", EDGE_CASES)
+def test_window_and_pooled_blocks_at_their_edges(hy, tmp_path, size, pool, n, decode_from):
+    """A small vocabulary and look-up heads: every query has earlier copies of its token at all distances, among them exactly at the
+    window's edge and in the block that is just seen or not yet, in the prompt and while decoding; key tiles are 64 wide, so sizes
+    around 64 and 128 put the edges on and next to the tiles' borders.  The restatement with a window one larger or smaller, or with
+    the blocks' edge moved by one position either way, differs by more than 10 times the bound (the token sequence is chosen so): a
+    kernel that is off by one cannot pass.  (With blocks of one position a key that leaves the window comes back as its own block: the
+    window's size alone then changes nothing, only the blocks' edge does.)"""
+    layers = [par(left=attn(heads=4, kv_heads=2, dim=16, vdim=24, scale=0.5, size=size, pool=pool, rot_dims=8), right=ret(heads=2, dim=12, vdim=8, rot_dims=4), ff=0),
+              par(left=attn(heads=2, kv_heads=2, dim=12, vdim=16, scale=0.3, size=size + 7, pool=max(1, pool - 1), rot_dims=4), ff=16)]
+    m = Model(hy, tmp_path, config(layers, width=64, vocab=97), seed=n, tweak=lookup_heads)
+
+    def sensitive(toks, ref):
+        knobs = [{"pool_shift": -1}, {"pool_shift": 1}] + ([{"size_delta": -1}, {"size_delta": 1}] if pool > 1 else [])
+        return all(err(m.ref(toks, **knob), ref) > 10 * F32_TOL for knob in knobs)
+
+    for seed in range(8):
+        toks, ref = m.tokens(n, seed=seed, vocab=23)
+        if sensitive(toks, ref):
+            break
+    else:
+        raise AssertionError("no token sequence shows every edge")
+    plan = m.plan("float32", ctx=n + 8, max_batch=96)
+    assert err(whole(plan, toks), ref) < F32_TOL
+    s = plan.acquire()
+    got = [plan.step(s, toks[:decode_from], 0, list(range(decode_from)))]
+    got += [plan.step(s, toks[i:i + 1], i, [0]) for i in range(decode_from, n)]
+    plan.release(s)
+    assert err(np.concatenate(got), ref) < F32_TOL
+    assert err(stepwise(plan, toks, [61, 2, 3, 64, 2, 67]), ref) < F32_TOL
+    plan.close()
+
+
+def test_far_tokens_reach_the_memories(hy, tmp_path):
+    """The first tokens of a long prompt decide the last logits only through the memories (the window and its pooled blocks are
+    switched off by a zero output projection of the attention): swapping two early tokens moves the restatement's last logits by far
+    more than the bound, and the plan follows, whole and decoded."""
+    layers = [par(left=attn(size=8, pool=4), right=ret(heads=2, dim=16, vdim=16, rot_dims=8, decay=[1.0, 0.999]), ff=0), mls(heads=2, dim=16, vdim=16, ff=0)]
+
+    def tweak(cfg, w):
+        w["l0.mix.left.o"] = np.zeros_like(w["l0.mix.left.o"])
+        w["l1.mix.f.b"] = np.full_like(w["l1.mix.f.b"], 9.0)        # forget gates near one
+
+    m = Model(hy, tmp_path, config(layers, width=48, vocab=61), seed=77, tweak=tweak)
+    n = 700
+    toks, ref = m.tokens(n)
+    other = toks.copy()
+    other[3], other[4] = (toks[3] + 1) % 61, (toks[4] + 7) % 61
+    assert err(m.ref(other)[-1:], ref[-1:]) > 20 * F32_TOL
+    plan = m.plan("float32", ctx=n, max_batch=256)
+    assert err(whole(plan, toks, [n - 1]), ref[-1:]) < F32_TOL
+    s = plan.acquire()
+    plan.step(s, toks[:n - 40], 0, [])
+    got = np.concatenate([plan.step(s, toks[i:i + 1], i, [0]) for i in range(n - 40, n)])
+    plan.release(s)
+    plan.close()
+    assert err(got, ref[n - 40:]) < F32_TOL
+
+
+def test_first_tokens(hy, tmp_path):
+    """Positions 0 .. 4 and a one-token sequence (through the decode kernels), with windows of 1 and 2 and blocks of 1 and 2."""
+    layers = [par(left=attn(size=2, pool=1), ff=0), mls(heads=2, dim=8, vdim=8), par(left=attn(heads=2, kv_heads=2, dim=8, vdim=8, size=1, pool=2, rot_dims=8))]
+    m = Model(hy, tmp_path, config(layers), seed=21, tweak=lookup_heads)
+    toks, ref = m.tokens(5, vocab=2)
+    plan = m.plan("float32", ctx=8)
+    assert err(whole(plan, toks), ref) < F32_TOL
+    assert err(whole(plan, toks[:1]), ref[:1]) < F32_TOL
+    assert err(stepwise(plan, toks, [1]), ref) < F32_TOL
+    assert err(stepwise(plan, toks, [2]), ref) < F32_TOL
+    plan.close()
+
+
+def test_long_decoding(hy, tmp_path):
+    layers = [par(left=attn(heads=2, kv_heads=1, dim=16, vdim=16, size=150, pool=6, rot_dims=16), right=ret(heads=2, dim=16, vdim=16, decay=[0.999, 0.96]), ff=16),
+              mls(heads=2, dim=8, vdim=8, ff=0), par(left=attn(heads=2, kv_heads=2, dim=8, vdim=8, size=33, pool=70, rot_dims=4), ff=0)]
+    m = Model(hy, tmp_path, config(layers, width=48, vocab=61), seed=33)
+    n = 420
+    toks, ref = m.tokens(n)
+    for dtype, tol in (("float32", F32_TOL), ("bfloat16", BF16_TOL)):
+        plan = m.plan(dtype, ctx=n)
+        s = plan.acquire()
+        plan.step(s, toks[:3], 0, [])
+        got = np.concatenate([plan.step(s, toks[i:i + 1], i, [0]) for i in range(3, n)])
+        plan.release(s)
+        plan.close()
+        assert err(got, ref[3:]) < tol, dtype
+
+
+def test_rotation_is_by_position_not_by_place_in_the_step(hy, tmp_path):
+    """Keys and queries of both mixers turn by the token's position in the sequence: with small bases and no position scaling the turns
+    are large, and a portion that starts late must turn by its true positions."""
+    m = Model(hy, tmp_path, config([par(left=attn(rot_dims=24, base=3.0, factor=None, size=200, pool=0, scale=1.0), right=ret(rot_dims=16, base=2.0))]), seed=61)
+    toks, ref = m.tokens(70)
+    plan = m.plan("float32", ctx=80)
+    assert err(stepwise(plan, toks, [33, 2, 1, 20, 14]), ref) < F32_TOL
+    plan.close()
+
+
+# ---- the framework's own entry points ------------------------------------------------------------------------------------------------------
+def check_greedy(m, prompt, ids):
+    """Every generated id is the reference's arg max given the ids before it (ties within 1e-4 of the maximum are allowed)."""
+    full = list(prompt) + list(ids)
+    ref = m.ref(np.array(full[:-1], np.int32))
+    for i, t in enumerate(ids):
+        row = ref[len(prompt) - 1 + i]
+        assert row[t] >= row.max() - 1e-4 * max(1.0, abs(row.max())), i
+
+
+def test_greedy_generation_python_entry(hy, tmp_path):
+    m = Model(hy, tmp_path, config(MIXED), seed=51)
+    prompt, _ = m.tokens(37)
+    plan = m.plan("float32", ctx=64, max_batch=16)
+    ids = plan.generate(prompt, 20)
+    check_greedy(m, prompt, ids)
+    plan.prefill(prompt[:-1], 0)
+    lg = plan.forward_decode(int(prompt[-1]), len(prompt) - 1)
+    assert int(np.argmax(lg)) == ids[0]
+    plan.prefill(prompt[:-1], 0)
+    t = plan.forward_decode_sample(int(prompt[-1]), len(prompt) - 1, 0.7, 0.9, 0.3)
+    assert 0 <= t < m.cfg["vocab"]
+    plan.close()
+
+
+def test_greedy_generation_command_line(hy, tmp_path):
+    m = Model(hy, tmp_path, config(MIXED), seed=52)
+    prompt, _ = m.tokens(21)
+    exe = os.path.join(ge.ROOT, "tools", "gl3_run")
+    out = subprocess.run([exe, "-m", m.dir, "--ids", ",".join(map(str, prompt)), "-n", "40", "-b", "8", "--f32"], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stderr
+    ids = [int(x) for x in out.stdout.split("generated:")[1].split()]
+    assert len(ids) == 40 - len(prompt) + 1
+    check_greedy(m, prompt, ids)
+
+
+def test_trace_replay_tool(hy, tmp_path):
+    m = Model(hy, tmp_path, config(MIXED[:3]), seed=53)
+    toks, ref = m.tokens(50)
+    outdir = tmp_path / "out"
+    outdir.mkdir()
+    steps = [{"step": 0, "entries": [{"id": "x", "tokens": toks[:30].tolist(), "want": [3, 29]}], "end": []},
+             {"step": 1, "entries": [{"id": "x", "tokens": toks[30:32].tolist(), "want": []}], "end": []},
+             {"step": 2, "entries": [{"id": "x", "tokens": toks[32:].tolist(), "want": [17]}], "end": ["x"]},
+             {"step": 3, "entries": [{"id": "y", "tokens": toks[:5].tolist(), "want": [4]}], "end": ["y"]}]
+    for dtype, tol in (("float32", F32_TOL), ("bfloat16", BF16_TOL)):
+        p = subprocess.run([os.path.join(ge.ROOT, "bin", "trace_run"), "--model", m.dir, "--dtype", dtype, "--out", str(outdir), "--max-tokens", "64"],
+                           input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=300)
+        assert p.returncode == 0, p.stderr
+        assert [l for l in p.stdout.split("\n") if l.startswith("done")] == ["done 0", "done 1", "done 2", "done 3"]
+        assert not (outdir / "1.f32").exists()
+        got = np.concatenate([np.fromfile(outdir / ("%d.f32" % i), np.float32).reshape(-1, m.cfg["vocab"]) for i in (0, 2, 3)])
+        assert err(got, ref[[3, 29, 49, 4]]) < tol
+
+
+def test_loader_refuses_what_it_cannot_run(hy, tmp_path):
+    m = Model(hy, tmp_path, config([par(), mls()]), seed=54)
+    for name in ("l0.mix.left.sink", "l0.mix.left.k.b", "l0.mix.left.q.norm", "l0.mix.right.g", "l0.mix.right.o", "l1.mix.f.b", "l1.mix.norm", "l1.mlp.up", "l0.norm1"):
+        w = dict(m.w)
+        del w[name]
+        hy.save_model_dir(str(tmp_path / "bad"), m.cfg, w)
+        with pytest.raises(hy.hip.Gl3Error):
+            hy.HybridPlan.from_dir(str(tmp_path / "bad"))
+    w = dict(m.w)
+    w["l0.mix.left.sink"] = np.concatenate([w["l0.mix.left.sink"], w["l0.mix.left.sink"]])
+    hy.save_model_dir(str(tmp_path / "bad"), m.cfg, w)
+    with pytest.raises(hy.hip.Gl3Error):
+        hy.HybridPlan.from_dir(str(tmp_path / "bad"))
+    for path, value in ((("left", "rot", "dims"), 7), (("right", "decay"), [0.5]), (("left", "kv_heads"), 3)):
+        bad = copy.deepcopy(m.cfg)
+        node = bad["layers"][0]["mixer"]
+        for key in path[:-1]:
+            node = node[key]
+        node[path[-1]] = value
+        hy.save_model_dir(str(tmp_path / "bad"), bad, m.w)
+        with pytest.raises(hy.hip.Gl3Error):
+            hy.HybridPlan.from_dir(str(tmp_path / "bad"))
