@@ -111,11 +111,17 @@ def main():
                     "per-layer token input, depth average): prefill and decode throughput at layer sizes of a real model beside the family's closest "
                     "design at equal size (Noditar attention layers with a dense feed-forward of the same active width); comma list of sizes from "
                     "1b,8b; prints its own JSON line instead of the tg/pp line")
+    ap.add_argument("--kosusun", default="", help="layer-list family, Kosusun design (bfloat16: parallel blocks; attention with pooled blocks behind a window "
+                    "beside retention; mLSTM layers): prefill and decode throughput at layer sizes of a real model beside the family's closest design at "
+                    "equal size (Noditar attention and state-space layers, same heads, state sizes and feed-forward); comma list of sizes from 1b,8b; "
+                    "prints its own JSON line instead of the tg/pp line")
     args = ap.parse_args()
     if args.hybrid:
         return bench_hybrid(args)
     if args.vonulix:
         return bench_vonulix(args)
+    if args.kosusun:
+        return bench_kosusun(args)
 
     if args.gpus > 1 and "WORLD_SIZE" not in os.environ:
         return self_spawn(args.gpus)
@@ -694,6 +700,54 @@ def vonulix_twin_config(z):
 def bench_vonulix(args):
     """Prefill (pp<n-prompt>, one step, no logits) and decode (tg<n-gen> from position 0 and from --depth positions, logits to the host every
     step) of the Vonulix design in bfloat16 beside the twin above."""
+    return bench_design_pair(args, "vonulix", "Vonulix", args.vonulix, VONULIX_SIZES, vonulix_config, vonulix_twin_config,
+                             "twin = Noditar attention layers with a dense feed-forward of the same active width, equal width / heads / layers / vocabulary")
+
+
+KOSUSUN_SIZES = {   # width, feed-forward, layers (parallel, parallel, mlstm, mlstm, ...), vocabulary; attention heads / kv heads / head size, window, block;
+                    # retention heads x key size x value size; mLSTM heads x key size x value size
+    "1b": dict(width=2048, ff=8192, n_layers=8, vocab=32000, heads=32, kv_heads=8, dim=64, window=1024, pool=16, r_heads=16, r_dim=64, r_vdim=128,
+               m_heads=8, m_dim=128, m_vdim=256),
+    "8b": dict(width=4096, ff=14336, n_layers=4, vocab=32000, heads=32, kv_heads=8, dim=128, window=1024, pool=16, r_heads=16, r_dim=128, r_vdim=256,
+               m_heads=8, m_dim=256, m_vdim=512),
+}
+
+
+def kosusun_config(z):
+    W, H, G, D = z["width"], z["heads"], z["kv_heads"], z["dim"]
+    mlp = {"kind": "dense", "ff": z["ff"]}
+    par = {"type": "parallel", "mlp": mlp,
+           "mixer": {"left": {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "scale": D ** -0.5, "mask": {"size": z["window"], "pool": z["pool"]},
+                              "rot": {"base": 500000.0, "dims": D, "scaling": {"factor": 2.0}}},
+                     "right": {"heads": z["r_heads"], "dim": z["r_dim"], "vdim": z["r_vdim"], "rot": {"base": 10000.0, "dims": z["r_dim"]},
+                               "decay": [1.0 - 2.0 ** (-5.0 - 3.0 * i / max(1, z["r_heads"] - 1)) for i in range(z["r_heads"])]},
+                     "left_scale": 0.7, "right_scale": 0.7}}
+    mls = {"type": "mlstm", "mlp": mlp, "mixer": {"heads": z["m_heads"], "dim": z["m_dim"], "vdim": z["m_vdim"], "gate_cap": 15.0}}
+    kinds = [par, par, mls, mls]
+    return {"architecture": "Kosusun", "vocab": z["vocab"], "width": W, "embedding": {"scale": float(W) ** 0.5}, "norm": {"eps": 1e-6}, "residual_mult": 0.5,
+            "logit_scale": 0.5, "layers": [kinds[i % 4] for i in range(z["n_layers"])]}
+
+
+def kosusun_twin_config(z):
+    """The family's closest design at equal size: Noditar layers on one stream — where Kosusun has attention beside retention, attention
+    with the same heads (no window, gated); where it has an mLSTM, the state-space mixer with the same heads, state rows (= key size) and
+    head width (= value size); the same feed-forward in every layer."""
+    W, H, G, D = z["width"], z["heads"], z["kv_heads"], z["dim"]
+    mlp = {"kind": "dense", "ff": z["ff"], "limit": 7.0}
+    att = {"type": "attention", "mixer": {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "scale": D ** -0.5}, "mlp": mlp}
+    ssm = {"type": "mamba2", "mixer": {"heads": z["m_heads"], "vdim": z["m_vdim"], "state": z["m_dim"], "groups": z["m_heads"], "norm_groups": z["m_heads"], "conv": 4}, "mlp": mlp}
+    kinds = [att, att, ssm, ssm]
+    return {"architecture": "Noditar", "vocab": z["vocab"], "width": W, "streams": 1, "norm": {"eps": 1e-5}, "layers": [kinds[i % 4] for i in range(z["n_layers"])]}
+
+
+def bench_kosusun(args):
+    """As bench_vonulix, for the Kosusun design beside its twin."""
+    return bench_design_pair(args, "kosusun", "Kosusun", args.kosusun, KOSUSUN_SIZES, kosusun_config, kosusun_twin_config,
+                             "twin = Noditar attention and state-space layers on one stream with the same heads, state sizes and feed-forward, equal width / "
+                             "layers / vocabulary")
+
+
+def bench_design_pair(args, label_key, design, sizes_arg, SIZES, config_fn, twin_fn, twin_text):
     import shutil
     import tempfile
     import numpy as np
@@ -716,13 +770,13 @@ def bench_vonulix(args):
         torch.cuda.synchronize()
         return (time.perf_counter() - t) / steps
 
-    for size in [x for x in args.vonulix.split(",") if x]:
-        z = VONULIX_SIZES[size]
+    for size in [x for x in sizes_arg.split(",") if x]:
+        z = SIZES[size]
         ctx = max([args.n_prompt] + depths) + args.n_gen + 8
         toks = np.asarray(pkg.javarand.bench_tokens(z["vocab"], ctx), np.int32)
         row = {"size": size, "shape": z}
-        for label, cfg in (("vonulix", vonulix_config(z)), ("twin", vonulix_twin_config(z))):
-            tmp = tempfile.mkdtemp(prefix="gl3_vonulix_")
+        for label, cfg in ((label_key, config_fn(z)), ("twin", twin_fn(z))):
+            tmp = tempfile.mkdtemp(prefix="gl3_%s_" % label_key)
             try:
                 hybrid.random_model_dir(tmp, cfg, seed=args.seed)
                 plan = hybrid.HybridPlan.from_dir(tmp, dtype="bfloat16", ctx=ctx, max_batch=args.batch)
@@ -749,12 +803,11 @@ def bench_vonulix(args):
         rows.append(row)
     head = rows[0]
     print(json.dumps({
-        "metric": "tg%d tok/s, Vonulix-design bf16 at %s layer sizes" % (args.n_gen, head["size"]), "value": head["vonulix"]["tg_tok_s"], "unit": "tok/s", "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(args.n_gen / head["vonulix"]["tg_tok_s"] * 1e3, 3), "higher_is_better": True,
+        "metric": "tg%d tok/s, %s-design bf16 at %s layer sizes" % (args.n_gen, design, head["size"]), "value": head[label_key]["tg_tok_s"], "unit": "tok/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(args.n_gen / head[label_key]["tg_tok_s"] * 1e3, 3), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": "random-weight Vonulix-design models (layer-list family), pp%d in one step without logits, tg%d with the logits copied to the "
-                               "host every step; twin = Noditar attention layers with a dense feed-forward of the same active width, equal width / heads / "
-                               "layers / vocabulary" % (args.n_prompt, args.n_gen), "parallelism": "single GPU"},
+        "config": {"workload": "random-weight %s-design models (layer-list family), pp%d in one step without logits, tg%d with the logits copied to the "
+                               "host every step; %s" % (design, args.n_prompt, args.n_gen, twin_text), "parallelism": "single GPU"},
         "sizes": rows}))
 
 

@@ -492,14 +492,21 @@ static __global__ __launch_bounds__(64) void hy_attn_prep_kernel(float* __restri
 
 // 1 / sqrt(mean((x + bias)^2) + eps) over two column ranges of every token's projection row (the whole q projection and the whole k
 // projection): out[2 t], out[2 t + 1].  Runs before the cache writers rewrite q in place.
-static __global__ __launch_bounds__(256) void hy_rowrms_kernel(const float* __restrict__ proj, int ld, int off0, int len0, int off1, int len1,
-                                                               const float* __restrict__ bias, float eps, float* __restrict__ out) {
-    __shared__ float red[4];
+template <int NT>
+static __global__ __launch_bounds__(NT) void hy_rowrms_kernel(const float* __restrict__ proj, int ld, int off0, int len0, int off1, int len1,
+                                                              const float* __restrict__ bias, float eps, float* __restrict__ out) {
+    __shared__ float red[NT / 64];
     const int t = blockIdx.x, which = blockIdx.y, off = which ? off1 : off0, len = which ? len1 : len0;
     const float* row = proj + (size_t)t * ld + off;
     float ss = 0.f;
-    for (int d = threadIdx.x; d < len; d += 256) { const float v = row[d] + (bias ? bias[off + d] : 0.f); ss += v * v; }
-    ss = hy_block_sum<256>(ss, red);
+    for (int d0 = threadIdx.x; d0 < len; d0 += 4 * NT) {          // four loads (and their biases) in flight per thread
+        float v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) { const int d = d0 + u * NT; v[u] = d < len ? row[d] + (bias ? bias[off + d] : 0.f) : 0.f; }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) ss += v[u] * v[u];
+    }
+    ss = hy_block_sum<NT>(ss, red);
     if (threadIdx.x == 0) out[2 * t + which] = 1.f / sqrtf(ss / (float)len + eps);
 }
 
@@ -514,9 +521,17 @@ static __global__ __launch_bounds__(256) void hy_pool_kernel(const float* __rest
     const int ld = blockIdx.y ? ldv : ldk;
     const float* src = (blockIdx.y ? vc : kc) + slot + (size_t)b * P * ld;
     float* dst = (blockIdx.y ? pv : pk) + slot + (size_t)b * ld;
-    for (int c = threadIdx.x; c < ld; c += 256) {
+    for (int c = blockIdx.z * 256 + threadIdx.x; c < ld; c += 256 * gridDim.z) {
         float a = 0.f;
-        for (int j = 0; j < P; ++j) a += src[(size_t)j * ld + c];
+        int j = 0;
+        for (; j + 8 <= P; j += 8) {          // eight rows in flight, added in position order
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = src[(size_t)(j + u) * ld + c];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) a += v[u];
+        }
+        for (; j < P; ++j) a += src[(size_t)j * ld + c];
         dst[c] = a / (float)P;
     }
 }
@@ -1038,19 +1053,36 @@ static __global__ __launch_bounds__(256) void hy_mem_gates_kernel(const float* _
 // head), divided by max(|y[V]|, ge[t][head]) + 1e-6 where the memory has a normaliser (ge != null); then o / sqrt(mean(o^2) + eps), times
 // w[head V + c] (null = none), times act(gate[t][g_off + head V + c]) (act = silu, or sigmoid for gate_act 1), times out_mul, stored in the
 // matrix type at out[t ldo + head V + c].
-template <typename TO>
-static __global__ __launch_bounds__(64) void hy_mem_out_kernel(const float* __restrict__ y, int ldy, int P, int V, const float* __restrict__ ge, int heads,
+// NT threads per (token, head): 64 for portions of many tokens, 256 for a few (a thread's column loop is a chain of load round trips).
+template <typename TO, int NT>
+static __global__ __launch_bounds__(NT) void hy_mem_out_kernel(const float* __restrict__ y, int ldy, int P, int V, const float* __restrict__ ge, int heads,
                                                                const float* __restrict__ w, const float* __restrict__ gate, int ldg, int g_off, int gate_act,
                                                                float eps, float out_mul, TO* __restrict__ out, int ldo) {
-    const int t = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+    __shared__ float red[NT / 64];
+    const int t = blockIdx.x, head = blockIdx.y, tid = threadIdx.x;
     const float* row = y + (size_t)t * ldy + (size_t)head * P;
     float inv = 1.f;
     if (ge) inv = 1.f / (fmaxf(fabsf(row[V]), ge[(size_t)t * heads + head]) + 1e-6f);
-    float ss = 0.f;
-    for (int c = lane; c < V; c += 64) { const float v = row[c] * inv; ss += v * v; }
-    ss = hy_wave_sum(ss);
+    // the first two columns of a thread stay in registers with their gate and weight (loaded before the sum's barrier)
+    float keep[2], kz[2], kw[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+        const int c = tid + u * NT;
+        keep[u] = c < V ? row[c] * inv : 0.f;
+        kz[u] = c < V ? gate[(size_t)t * ldg + g_off + head * V + c] : 0.f;
+        kw[u] = (c < V && w) ? w[head * V + c] : 1.f;
+    }
+    float ss = keep[0] * keep[0] + keep[1] * keep[1];
+    for (int c = tid + 2 * NT; c < V; c += NT) { const float v = row[c] * inv; ss += v * v; }
+    if constexpr (NT == 64) ss = hy_wave_sum(ss);
+    else ss = hy_block_sum<NT>(ss, red);
     const float r = 1.f / sqrtf(ss / (float)V + eps);
-    for (int c = lane; c < V; c += 64) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+        const int c = tid + u * NT;
+        if (c < V) hy_st(out + (size_t)t * ldo + head * V + c, keep[u] * r * kw[u] * (gate_act == 1 ? hy_sigmoid(kz[u]) : hy_silu(kz[u])) * out_mul);
+    }
+    for (int c = tid + 2 * NT; c < V; c += NT) {
         const float z = gate[(size_t)t * ldg + g_off + head * V + c];
         const float gv = gate_act == 1 ? hy_sigmoid(z) : hy_silu(z);
         hy_st(out + (size_t)t * ldo + head * V + c, row[c] * inv * r * (w ? w[head * V + c] : 1.f) * gv * out_mul);

@@ -760,14 +760,17 @@ static int32_t hy_mixer_core(gl3_ctx* ctx, HyLayer& L, int np, int ldo, int n, i
         float* pv = d.pool > 0 ? h->slots + L.off_pv : nullptr;
         const HyRot rot{d.rot_dims, L.rot_freq, d.v_unit_norm, d.v_rot ? L.vrot_freq : nullptr, d.rot_interleaved};
         const HyPrepX px{d.qk_bias ? L.pbias : nullptr, L.qn, L.kn, h->rowr};
-        if (d.qk_unit_norm == 2)
-            hipLaunchKernelGGL(hy_rowrms_kernel, dim3(n, 2), dim3(256), 0, st, h->proj, np, L.q_off, d.heads * d.dim, L.k_off, d.kv_heads * d.dim, px.bias, eps, h->rowr);
+        if (d.qk_unit_norm == 2) {
+            if (n <= 32) hipLaunchKernelGGL((hy_rowrms_kernel<1024>), dim3(n, 2), dim3(1024), 0, st, h->proj, np, L.q_off, d.heads * d.dim, L.k_off, d.kv_heads * d.dim, px.bias, eps, h->rowr);
+            else hipLaunchKernelGGL((hy_rowrms_kernel<256>), dim3(n, 2), dim3(256), 0, st, h->proj, np, L.q_off, d.heads * d.dim, L.k_off, d.kv_heads * d.dim, px.bias, eps, h->rowr);
+        }
         hipLaunchKernelGGL(hy_attn_prep_kernel, dim3(n, d.heads + 2 * d.kv_heads), dim3(64), 0, st, h->proj, np, L.q_off, L.k_off, L.v_off, d.heads, d.kv_heads, d.dim,
                            d.vdim, d.qk_unit_norm, eps, kc, vc, h->slot_floats, h->dyn, rot, px);
         if (d.pool > 0) {
             const int done = (pos0 + n) / d.pool - pos0 / d.pool;          // blocks whose last position lies in this portion
             if (done > 0)
-                hipLaunchKernelGGL(hy_pool_kernel, dim3(done, 2), dim3(256), 0, st, kc, vc, pk, pv, d.kv_heads * d.dim, d.kv_heads * d.vdim, d.pool, h->slot_floats, h->dyn, n);
+                hipLaunchKernelGGL(hy_pool_kernel, dim3(done, 2, done <= 8 ? std::min(16, hy_cdiv(d.kv_heads * std::max(d.dim, d.vdim), 256)) : 1), dim3(256), 0, st, kc, vc, pk, pv,
+                                   d.kv_heads * d.dim, d.kv_heads * d.vdim, d.pool, h->slot_floats, h->dyn, n);
         }
         int32_t r = hy_attention(ctx, h->proj + L.q_off, np, kc, vc, d.heads, d.kv_heads, d.dim, d.vdim, d.scale, d.slope_log2, n, pos0, &nsplit, true, d.window, d.keep_first,
                                  pk, pv, d.pool);
@@ -792,8 +795,12 @@ static int32_t hy_mixer_core(gl3_ctx* ctx, HyLayer& L, int np, int ldo, int n, i
         a.heads = d.heads; a.P = P; a.N = d.dim; a.G = d.heads;
         a.state = h->slots + L.off_state; a.slot_stride = h->slot_floats; a.dyn = h->dyn; a.n = n; a.y = h->ssm_y; a.ldy = ldy;
         hy_scan(ctx, a);
-        hipLaunchKernelGGL((hy_mem_out_kernel<T>), dim3(n, d.heads), dim3(64), 0, st, h->ssm_y, ldy, P, d.vdim, eg ? ge : nullptr, d.heads,
-                           d.mem_norm_weight ? L.ssm_norm : nullptr, h->proj, np, L.g_off, d.mem_gate_act, eps, L.out_mul, mixo, ldo);
+        if (n <= 32 && d.vdim > 128)
+            hipLaunchKernelGGL((hy_mem_out_kernel<T, 256>), dim3(n, d.heads), dim3(256), 0, st, h->ssm_y, ldy, P, d.vdim, eg ? ge : nullptr, d.heads,
+                               d.mem_norm_weight ? L.ssm_norm : nullptr, h->proj, np, L.g_off, d.mem_gate_act, eps, L.out_mul, mixo, ldo);
+        else
+            hipLaunchKernelGGL((hy_mem_out_kernel<T, 64>), dim3(n, d.heads), dim3(64), 0, st, h->ssm_y, ldy, P, d.vdim, eg ? ge : nullptr, d.heads,
+                               d.mem_norm_weight ? L.ssm_norm : nullptr, h->proj, np, L.g_off, d.mem_gate_act, eps, L.out_mul, mixo, ldo);
     } else if (d.mixer == GL3_MIX_LATENT) {
         float* cc = h->slots + L.off_k;
         const int R = d.kv_rank;

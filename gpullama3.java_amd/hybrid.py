@@ -1,4 +1,4 @@
-"""Host side of the layer-list family (GL3_ARCH_LAYERLIST: the Noditar and Vonulix designs) over the C-ABI: model folders (config.json + model.safetensors), the step
+"""Host side of the layer-list family (GL3_ARCH_LAYERLIST: the Noditar, Vonulix and Kosusun designs) over the C-ABI: model folders (config.json + model.safetensors), the step
 function with sequence slots, greedy / sampled generation.  The compute path is csrc/gl3_hybrid.hip; nothing here computes.
 
     plan = HybridPlan.from_dir("model-folder", dtype="bfloat16", ctx=4096, max_batch=512, n_seqs=2)
@@ -223,16 +223,45 @@ def vonulix_tensor_shapes(config: dict) -> dict:
     return out
 
 
+def kosusun_tensor_shapes(config: dict) -> dict:
+    """{tensor name: shape} of a Kosusun configuration, in file order."""
+    W, V = config["width"], config["vocab"]
+    out = {"embed": (V, W)}
+    for i, layer in enumerate(config["layers"]):
+        p, m, ff = "l%d." % i, layer["mixer"], layer.get("mlp")
+        out[p + "norm1"] = (W,)
+        if layer["type"] == "parallel":
+            a, r, q = m["left"], m["right"], p + "mix.left."
+            nq, nk, nv = a["heads"] * a["dim"], a["kv_heads"] * a["dim"], a["kv_heads"] * a["vdim"]
+            out.update({q + "q": (nq, W), q + "q.b": (nq,), q + "k": (nk, W), q + "k.b": (nk,), q + "v": (nv, W), q + "v.b": (nv,), q + "q.norm": (nq,),
+                        q + "k.norm": (nk,), q + "sink": (a["heads"],), q + "o": (W, a["heads"] * a["vdim"])})
+            q = p + "mix.right."
+            out.update({q + "q": (r["heads"] * r["dim"], W), q + "k": (r["heads"] * r["dim"], W), q + "v": (r["heads"] * r["vdim"], W),
+                        q + "g": (r["heads"] * r["vdim"], W), q + "o": (W, r["heads"] * r["vdim"])})
+        else:
+            q, od = p + "mix.", m["heads"] * m["vdim"]
+            out.update({q + "q": (m["heads"] * m["dim"], W), q + "k": (m["heads"] * m["dim"], W), q + "v": (od, W), q + "g": (od, W), q + "o": (W, od),
+                        q + "norm": (od,), q + "i": (m["heads"], W), q + "i.b": (m["heads"],), q + "f": (m["heads"], W), q + "f.b": (m["heads"],)})
+        if ff:
+            out.update({p + "mlp.gate": (ff["ff"], W), p + "mlp.up": (ff["ff"], W), p + "mlp.down": (W, ff["ff"])})
+    out["final.norm"] = (W,)
+    out["head"] = (V, W)
+    return out
+
+
 def random_model_dir(path: str, config: dict, seed: int = 0):
     """A model folder with random weights for timing: matrices are random bfloat16 bit patterns of magnitude 2^-9 .. 2^-6 / sqrt-free (cheap to
     make at billions of elements), vectors and tables are benign constants with noise."""
     rng = np.random.default_rng(seed)
     S = config.get("streams", 1)
     t = {}
-    vonulix = config["architecture"] == "Vonulix"
-    for name, shp in (vonulix_tensor_shapes(config) if vonulix else noditar_tensor_shapes(config)).items():
+    vonulix, kosusun = config["architecture"] == "Vonulix", config["architecture"] == "Kosusun"
+    shapes = vonulix_tensor_shapes(config) if vonulix else kosusun_tensor_shapes(config) if kosusun else noditar_tensor_shapes(config)
+    for name, shp in shapes.items():
         leaf = name.split(".", 1)[1] if name[0] == "l" and name[1].isdigit() else name
-        if vonulix and leaf in ("norm1", "norm2", "final.norm"):
+        if kosusun and leaf.endswith((".b", ".sink")):
+            t[name] = np.full(shp, 3.0 if leaf.endswith("f.b") else 0.0, np.float32)          # forget gates near one, no other offsets
+        elif vonulix and leaf in ("norm1", "norm2", "final.norm"):
             t[name] = np.zeros(shp, np.float32)                  # the file holds weight - 1
         elif leaf == "dwa":
             t[name] = np.concatenate([np.full(shp[0] - 1, 0.1 / max(1, shp[0] - 1)), [0.9]]).astype(np.float32)
