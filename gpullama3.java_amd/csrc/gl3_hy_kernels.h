@@ -886,8 +886,8 @@ static __global__ __launch_bounds__(256) void hy_conv_tail_kernel(const float* _
 // Recurrence S_t = a_t S_(t-1) + b_t k_t x_t^T,  y_t = S_t^T q_t + D x_t  per head, S = N x P (keys / queries of N entries, values of P).
 // Three sources of a_t, b_t (HyScanArgs.mode): 0, a state-space layer: dt = softplus(raw + bias), a = e^(-e^(A_log) dt), b = dt, keys
 // and queries shared by the heads of a group; 1, gates that a kernel before this one left per (token, head) (hy_mem_gates_kernel);
-// 2, a fixed decay per head, b = 1.  Keys and queries may turn by their position on the way into LDS (rot: first `dims` entries, pairs
-// (i, i + dims / 2) or (2 i, 2 i + 1), angle = position * freq[i]) and are multiplied by k_mul / q_mul afterwards.  ones_col: the last of
+// 2, a fixed decay per head, b = 1.  Keys and queries are multiplied by k_mul / q_mul on the way into LDS and may turn there by their
+// position (rot: first `dims` entries, pairs (i, i + dims / 2) or (2 i, 2 i + 1), angle = position * freq[i]).  ones_col: the last of
 // the P columns has x = 1 whatever the token (it then carries n_t = a n + b k, the normaliser of a matrix memory, and y's last column
 // is n_t . q_t).
 // Workgroup = one head x 4 wavefronts; a wavefront = 64 / NG value columns, a column's N states spread over NG lanes (lane i holds the NL
@@ -912,16 +912,36 @@ struct HyScanArgs {
     float* state; size_t slot_stride; const int* dyn; int n;
     float* y; int ldy;                                 // y of (t, head, column): y + t ldy + head P + column
 };
-__device__ __forceinline__ float hy_scan_fetch(const float* __restrict__ row, int nn, int N, const HyScanRot& rot, float pos) {
-    if (nn >= N) return 0.f;
-    if (nn >= rot.dims) return row[nn];
+// rows t0 .. t0 + tb - 1 (N floats each, row stride ld) times mul -> dst[t Ns + n], zero behind N; eight loads in flight per thread
+__device__ __forceinline__ void hy_scan_stage(float* __restrict__ dst, const float* __restrict__ base, int ld, int t0, int tb, int N, int Ns, float mul) {
+    const int total = tb * Ns;
+    for (int i0 = threadIdx.x; i0 < total; i0 += 8 * 256) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int i = i0 + u * 256, t = i / Ns, nn = i - t * Ns;
+            v[u] = (i < total && nn < N) ? base[(size_t)(t0 + t) * ld + nn] : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int i = i0 + u * 256;
+            if (i < total) dst[i] = v[u] * mul;
+        }
+    }
+}
+// the staged rows turn in place by their position: one thread per pair
+__device__ __forceinline__ void hy_scan_turn(float* __restrict__ rows, int tb, int Ns, const HyScanRot& rot, int pos) {
     const int half = rot.dims >> 1;
-    const int i = rot.interleaved ? nn >> 1 : (nn < half ? nn : nn - half);
-    const bool first = rot.interleaved ? !(nn & 1) : nn < half;
-    const int other = rot.interleaved ? nn ^ 1 : (first ? nn + half : nn - half);
-    float sn, cs;
-    sincosf(pos * rot.freq[i], &sn, &cs);
-    return first ? row[nn] * cs - row[other] * sn : row[nn] * cs + row[other] * sn;
+    for (int i = threadIdx.x; i < tb * half; i += 256) {
+        const int t = i / half, j = i - t * half;
+        const int i0 = rot.interleaved ? 2 * j : j, i1 = rot.interleaved ? 2 * j + 1 : j + half;
+        float sn, cs;
+        sincosf((float)(pos + t) * rot.freq[j], &sn, &cs);
+        float* r = rows + t * Ns;
+        const float u = r[i0], v = r[i1];
+        r[i0] = u * cs - v * sn;
+        r[i1] = v * cs + u * sn;
+    }
 }
 template <int NL>
 static __global__ __launch_bounds__(256) void hy_ssm_scan_kernel(HyScanArgs a) {
@@ -953,12 +973,8 @@ static __global__ __launch_bounds__(256) void hy_ssm_scan_kernel(HyScanArgs a) {
     for (int t0 = 0; t0 < n; t0 += TB) {
         const int tb = min(TB, n - t0);
         __syncthreads();
-        for (int i = tid; i < tb * Ns; i += 256) {
-            const int t = i / Ns, nn = i - t * Ns;
-            const float pos = (float)(pos0 + t0 + t);
-            sB[i] = hy_scan_fetch(kbase + (size_t)(t0 + t) * a.ldk, nn, N, a.rot, pos) * a.k_mul;
-            sC[i] = hy_scan_fetch(qbase + (size_t)(t0 + t) * a.ldq, nn, N, a.rot, pos) * a.q_mul;
-        }
+        hy_scan_stage(sB, kbase, a.ldk, t0, tb, N, Ns, a.k_mul);
+        hy_scan_stage(sC, qbase, a.ldq, t0, tb, N, Ns, a.q_mul);
         for (int i = tid; i < tb * cols; i += 256) {
             const int t = i / cols, c = i - t * cols;
             sX[i] = col0 + c < Px ? xbase[(size_t)(t0 + t) * a.ldx + col0 + c] : (col0 + c < P ? 1.f : 0.f);
@@ -975,6 +991,11 @@ static __global__ __launch_bounds__(256) void hy_ssm_scan_kernel(HyScanArgs a) {
                 sDt[tid] = 1.f;
                 sDt[TB + tid] = fixed;
             }
+        }
+        if (a.rot.dims > 0) {          // a turn is linear: the multiplier went in with the staging
+            __syncthreads();
+            hy_scan_turn(sB, tb, Ns, a.rot, pos0 + t0);
+            hy_scan_turn(sC, tb, Ns, a.rot, pos0 + t0);
         }
         __syncthreads();
         for (int t = 0; t < tb; ++t) {

@@ -728,8 +728,15 @@ static int32_t hy_attention(gl3_ctx* ctx, const float* q, int ldq, const float* 
 
 // The recurrence kernel: a column's states over NG lanes x NL registers: NL = 16 (32 for more than 1024 states, 8 / 4 for very small
 // ones), NG a power of two; tokens staged per round: what fits 48 KB of LDS, at most 32.  Fills in a.NG and a.TB.
+// With few workgroups (few heads, narrow values) NL = 16 is halved once so that more of them share the columns; below 8 every workgroup
+// stages the same key / query rows for too few columns and the traffic from L2 eats the gain (measured: 16 and 8 within 2 %, 4 slower).
+// GL3_HY_SCAN_NL forces a value.
 static void hy_scan(gl3_ctx* ctx, HyScanArgs& a) {
-    const int NL = a.N > 1024 ? 32 : a.N > 8 ? 16 : a.N > 4 ? 8 : 4;
+    int NL = a.N > 1024 ? 32 : a.N > 8 ? 16 : a.N > 4 ? 8 : 4;
+    auto wgs = [&](int nl) { int ng = 1; while (ng * nl < a.N) ng *= 2; return (long)hy_cdiv(a.P, 4 * (64 / ng)) * a.heads; };
+    if (NL == 16 && 8 * 64 >= a.N && wgs(16) < 512) NL = 8;
+    static const int env_nl = getenv("GL3_HY_SCAN_NL") ? atoi(getenv("GL3_HY_SCAN_NL")) : 0;
+    if ((env_nl == 4 || env_nl == 8 || env_nl == 16 || env_nl == 32) && env_nl * 64 >= a.N) NL = env_nl;
     int NG = 1;
     while (NG * NL < a.N) NG *= 2;
     const int cols = 4 * (64 / NG), Ns = NG * NL;

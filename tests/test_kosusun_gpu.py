@@ -81,11 +81,15 @@ class Model:
         return toks, self.ref(toks)
 
 
-def err(got, want):
+def err_rows(got, want):
     d = got - want
     d = d - d.mean(axis=-1, keepdims=True)
     w = want - want.mean(axis=-1, keepdims=True)
-    return float(np.sqrt((d ** 2).mean(axis=-1)).max() / np.sqrt((w ** 2).mean()))
+    return np.sqrt((d ** 2).mean(axis=-1)) / np.sqrt((w ** 2).mean())
+
+
+def err(got, want):
+    return float(err_rows(got, want).max())
 
 
 def whole(plan, toks, want=None):
@@ -181,6 +185,48 @@ def test_layer_taps(hy, tmp_path):
         assert np.abs(rows - t).max() < 1e-4 * max(1.0, np.abs(t).max()), l
     plan.close()
     assert err(got, ref) < F32_TOL
+
+
+def random_config(seed):
+    """Layer order, every size and every constant drawn at random (sizes that are no multiples of anything included)."""
+    rng = np.random.default_rng(seed)
+    pick = lambda *xs: xs[int(rng.integers(len(xs)))]
+    layers = []
+    for _ in range(int(rng.integers(2, 6))):
+        ff = pick(0, int(rng.integers(8, 90)))
+        if rng.random() < 0.6:
+            G = pick(1, 2, 3)
+            D, Dr = 2 * int(rng.integers(2, 20)), 2 * int(rng.integers(1, 16))
+            left = attn(heads=G * pick(1, 2, 4), kv_heads=G, dim=D, vdim=int(rng.integers(3, 50)), scale=float(rng.uniform(0.1, 0.6)), size=int(rng.integers(1, 90)),
+                        pool=pick(0, 1, int(rng.integers(2, 40))), rot_dims=2 * int(rng.integers(1, D // 2 + 1)), base=float(rng.uniform(5.0, 1e5)),
+                        factor=pick(None, float(rng.uniform(1.0, 8.0))))
+            Hr = int(rng.integers(1, 6))
+            right = ret(heads=Hr, dim=Dr, vdim=int(rng.integers(2, 40)), rot_dims=2 * int(rng.integers(1, Dr // 2 + 1)), base=float(rng.uniform(5.0, 1e6)),
+                        decay=[float(1.0 - 2.0 ** -rng.uniform(1.0, 9.0)) for _ in range(Hr)])
+            layers.append(par(left=left, right=right, ff=ff, ls=float(rng.uniform(0.3, 1.5)), rs=float(rng.uniform(0.3, 1.5))))
+        else:
+            layers.append(mls(heads=int(rng.integers(1, 6)), dim=int(rng.integers(2, 40)), vdim=int(rng.integers(2, 50)), cap=float(rng.uniform(1.0, 20.0)), ff=ff))
+    return config(layers, width=int(rng.integers(20, 140)), vocab=int(rng.integers(30, 300)), emb_scale=float(rng.uniform(0.5, 6.0)), eps=float(10.0 ** -rng.uniform(4, 7)),
+                  mult=float(rng.uniform(0.3, 1.2)), logit_scale=float(rng.uniform(0.2, 2.0)))
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_configurations(hy, tmp_path, seed):
+    m = Model(hy, tmp_path, random_config(seed), seed=100 + seed)
+    n = 140
+    toks, ref = m.tokens(n, seed=seed)
+    # float32 holds every position to the bound.  bfloat16: a drawn configuration may hold a position where a small head's output nearly
+    # vanishes before its unit-RMS norm, which amplifies the rounding of the products' inputs without limit (the restatement with its
+    # inputs rounded alike has its worst row at the same position): nineteen rows in twenty are held to the bound, the median to a third
+    for dtype in ("float32", "bfloat16"):
+        plan = m.plan(dtype, ctx=n + 4, max_batch=48)
+        for got in (whole(plan, toks), stepwise(plan, toks, [50, 2, 1, 31, 7, 1])):
+            if dtype == "float32":
+                assert err(got, ref) < F32_TOL
+            else:
+                rows = err_rows(got, ref)
+                assert np.quantile(rows, 0.95) < BF16_TOL and np.median(rows) < BF16_TOL / 3
+        plan.close()
 
 
 # ---- prompts cut into portions, decoding token by token -----------------------------------------------------------------------------------
