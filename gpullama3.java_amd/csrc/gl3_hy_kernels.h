@@ -510,8 +510,8 @@ static __global__ __launch_bounds__(NT) void hy_rowrms_kernel(const float* __res
     if (threadIdx.x == 0) out[2 * t + which] = 1.f / sqrtf(ss / (float)len + eps);
 }
 
-// Pooled rows of a cache: block b holds positions b P .. b P + P - 1 and its pooled key / value is the mean of the block's cached rows
-// (summed in position order).  One workgroup per block that the step completes (its last position lies in the step) and cache
+// Pooled rows of a cache: the P cached rows of run b (positions b P .. b P + P - 1) are averaged into pooled row b (summed in position
+// order).  One workgroup per block that the step completes (its last position lies in the step) and cache
 // (blockIdx.y = 0 keys, 1 values).
 static __global__ __launch_bounds__(256) void hy_pool_kernel(const float* __restrict__ kc, const float* __restrict__ vc, float* __restrict__ pk, float* __restrict__ pv,
                                                              int ldk, int ldv, int P, size_t slot_stride, const int* __restrict__ dyn, int n) {

@@ -335,7 +335,7 @@ bool vonulix_tensor(const std::string& name, int32_t& id, int32_t& layer, int32_
 // Kosusun: every layer is a parallel block — one RMS norm, whose output feeds the mixer and the feed-forward alike, and
 // x <- x + residual_mult (mixer + feed-forward).  Two layer types.  "parallel": two mixers side by side, `left` = grouped-query attention
 // (biased q / k / v, RMS norm with weights over the whole q and the whole k projection, interleaved rotary pairs with linear position
-// scaling, a sliding window plus the means of the blocks of `mask.pool` positions that lie wholly before it, a learned sink logit per
+// scaling, a sliding window plus one averaged key / value per finished run of `mask.pool` positions behind it, a learned sink logit per
 // head) and `right` = retention (a matrix memory with a fixed decay per head, half-split rotary pairs, keys times dim^(-1/2), unit-RMS
 // heads times silu(W_g h)), added as left_scale * left + right_scale * right.  "mlstm": a matrix memory with exponential gates
 // (capped log gates, running maximum, normaliser; queries times dim^(-1/2); unit-RMS heads with a weight, times sigmoid(W_g h)).  The

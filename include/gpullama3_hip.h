@@ -127,13 +127,14 @@ typedef struct gl3_layer_desc {
     float   shared_limit;
     int32_t ff_act;             /* 0: act = g sigmoid(ff_alpha g) (u + ff_shift); 1: act = gelu_tanh(g) u */
     /* attention, further switches (each usable alone).  qk_bias: q, k and v projections have biases (GL3_T_BQ / BK / BV).
-     * qk_unit_norm = 2: RMS norm over the WHOLE q projection (all heads at once) and the whole k projection, with plain weights
+     * qk_unit_norm = 2: ONE root mean square for the token's whole q row (every head together), another for its whole k row, times the weights
      * GL3_T_ATTN_Q_NORM [heads dim] / GL3_T_ATTN_K_NORM [kv_heads dim], after the bias and before the rotation.  rot_interleaved:
      * rotary pairs are entries (2 i, 2 i + 1) instead of (i, i + rot_dims / 2) (also read by a matrix memory).  softmax_sink = 2: a
      * learned logit per head (GL3_T_ATTN_SINK [heads]) joins the denominator as e^sink, unscaled, without key or value.
-     * pool > 0 (needs window > 0): beside the window's keys, query i sees one key / value per block of `pool` positions that lies
-     * wholly before its window (block b = positions b pool .. b pool + pool - 1, seen if b pool + pool - 1 <= i - window): the means of
-     * the block's cached keys and values; positions between the seen blocks and the window are not seen at all */
+     * pool > 0 (needs window > 0): older context reaches query i in averaged form.  The cache is cut into runs of `pool` consecutive
+     * positions; a run whose LAST position is <= i - window contributes one extra key / value to the query's softmax, the arithmetic
+     * mean of the run's cached key rows / value rows.  A position that is outside the window and whose run is not finished that far
+     * back contributes nothing */
     int32_t qk_bias, rot_interleaved, pool;
     /* matrix memory (GL3_MIX_MEMORY): heads, dim (keys / queries), vdim; rot_* turn q and k as in attention; q and k are multiplied by
      * mem_q_mul / mem_k_mul (0 = 1) after the rotation.  The head's output is divided by its root mean square, multiplied by the weight

@@ -72,8 +72,8 @@ def blocks_seen(i, size, pool, shift=0):
 
 def pooled_window_attention(h, p, c, eps, size_delta=0, pool_shift=0):
     """Grouped-query attention: biased q / k / v, RMS norm with weights over the whole q and the whole k projection, interleaved rotary
-    pairs, a window of mask.size positions, one key / value (the mean) per block of mask.pool positions wholly before the window, a
-    learned sink logit per head in the denominator."""
+    pairs, a window of mask.size positions, one averaged key / value per finished block of mask.pool positions behind the window (see
+    blocks_seen), a learned sink logit per head in the denominator."""
     T = h.shape[0]
     H, G, D, V = c["heads"], c["kv_heads"], c["dim"], c["vdim"]
     mask = c.get("mask") or {}
