@@ -37,8 +37,7 @@ def test_product_path_never_touches_the_oracle():
                 src = open(os.path.join(root, f), errors="ignore").read()
                 assert not pat.search(src), f
     so = os.path.join(ge.PKG_DIR, "libgpullama_hip.so")
-    needed = subprocess.run(["readelf", "-d", so], capture_output=True, text=True).stdout
-    assert "oracle" not in needed
+    assert b"libgl3_oracle" not in open(so, "rb").read()          # no dependency on the oracle library
 
 
 def test_create_rejects_bad_descriptors_without_a_gpu(pkg):
