@@ -148,13 +148,15 @@ static __global__ __launch_bounds__(NT) void hy_streams_kernel(float* __restrict
 // ---- GEMM: C[m][n] = sum_k A[m][k] W[n][k]  (tokens x features, both operands K-contiguous) --------------------------------------
 typedef float hy_v16f __attribute__((ext_vector_type(16)));
 
-// Epilogues: STORE = the float32 products; GLU = gate / up pairs -> activation in the matrix type; ACTMUL = gelu_tanh(product) times an
-// entry of a per-token table row (mul_table[mul_rows[m]][mul_col0 + feature]) in the matrix type (the per-layer token input).
+// Epilogues: STORE = the float32 products; GLU = gate / up pairs -> activation in the matrix type; ACTMUL = act(product) in the matrix
+// type: gelu_tanh(product) times an entry of a per-token table row (mul_table[mul_rows[m]][mul_col0 + feature], the per-layer token
+// input), or relu(product)^2 alone (act = 2, mul_table = null: a feed-forward without a gate).
 enum { HY_EPI_STORE = 0, HY_EPI_GLU = 1, HY_EPI_ACTMUL = 2 };
-struct HyGlu { float limit, alpha, shift; const void* mul_table; const int* mul_rows; int mul_ld, mul_col0; int act; };      // act 1: gelu_tanh(g) u
+struct HyGlu { float limit, alpha, shift; const void* mul_table; const int* mul_rows; int mul_ld, mul_col0; int act; };      // act 1: gelu_tanh(g) u; 2: relu(u)^2, no gate
 __device__ __forceinline__ float hy_gelu_tanh(float z) { return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z))); }
 template <typename T>
 __device__ __forceinline__ float hy_actmul(float a, int m, int feature, const HyGlu& p) {
+    if (p.act == 2) { const float r = fmaxf(a, 0.f); return r * r; }
     return hy_gelu_tanh(a) * hy_ld((const T*)p.mul_table + (size_t)p.mul_rows[m] * p.mul_ld + p.mul_col0 + feature);
 }
 __device__ __forceinline__ float hy_glu(float g, float u, const HyGlu& p) {
@@ -549,13 +551,73 @@ static __global__ __launch_bounds__(64) void hy_latent_norm_kernel(const float* 
     for (int r = lane; r < R; r += 64) dst[r] = src[r] * s * cnorm[r];
 }
 
-// Per-head products out[t][h][c] = sum_k in[t][h][k] Wt[h][k][c] (float32), optionally times sigmoid(gate[t][h][c]), for portions of a
+// Latent attention with a rotated part (D unrotated + P rotated entries per query head, one rotated key part of P entries for all heads,
+// cached behind the latent).  blockIdx.y = 0: the first R entries of the token's down projection are RMS-normed with their weight into
+// the slot row's [0, R), the P entries behind them turn by the position into [R, R + P) (nothing when cc == null: a layer that reads
+// another layer's cache).  blockIdx.y = 1 + h: the last P entries of query head h turn in place.  Turn: pair (i, i + P / 2) becomes
+// (u c - v s, v c + u s), c = mscale cos(pos freq[i]), s = mscale sin(pos freq[i]).
+static __global__ __launch_bounds__(64) void hy_latent_prep_kernel(float* __restrict__ q, int ldq, int D, int P, const float* __restrict__ proj, int ld, int c_off, int R,
+                                                                   const float* __restrict__ cnorm, float eps, float* __restrict__ cc, size_t slot_stride,
+                                                                   const int* __restrict__ dyn, const float* __restrict__ freq, float mscale) {
+    const int t = blockIdx.x, lane = threadIdx.x, half = P >> 1;
+    const float pos = (float)(dyn[0] + t);
+    if (blockIdx.y == 0) {
+        if (!cc) return;
+        const float* src = proj + (size_t)t * ld + c_off;
+        float ss = 0.f;
+        for (int r = lane; r < R; r += 64) ss += src[r] * src[r];
+        ss = hy_wave_sum(ss);
+        const float s = 1.f / sqrtf(ss / (float)R + eps);
+        float* dst = cc + (size_t)dyn[1] * slot_stride + (size_t)(dyn[0] + t) * (R + P);
+        for (int r = lane; r < R; r += 64) dst[r] = src[r] * s * cnorm[r];
+        for (int i = lane; i < half; i += 64) {
+            float sn, cs;
+            sincosf(pos * freq[i], &sn, &cs);
+            sn *= mscale; cs *= mscale;
+            const float u = src[R + i], v = src[R + half + i];
+            dst[R + i] = u * cs - v * sn;
+            dst[R + half + i] = v * cs + u * sn;
+        }
+    } else {
+        float* qr = q + (size_t)t * ldq + (size_t)(blockIdx.y - 1) * (D + P) + D;
+        for (int i = lane; i < half; i += 64) {
+            float sn, cs;
+            sincosf(pos * freq[i], &sn, &cs);
+            sn *= mscale; cs *= mscale;
+            const float u = qr[i], v = qr[half + i];
+            qr[i] = u * cs - v * sn;
+            qr[half + i] = v * cs + u * sn;
+        }
+    }
+}
+
+// out[t][0 .. len) = rms_norm(src[t][off .. off + len)) * w in the matrix type (the operand of a following product); one workgroup per token
+template <typename TO>
+static __global__ __launch_bounds__(256) void hy_rownorm_kernel(const float* __restrict__ src, int ld, int off, int len, const float* __restrict__ w, float eps,
+                                                                TO* __restrict__ out, int ldo) {
+    __shared__ float red[4];
+    const int t = blockIdx.x;
+    const float* row = src + (size_t)t * ld + off;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < len; i += 256) ss += row[i] * row[i];
+    ss = hy_block_sum<256>(ss, red);
+    const float r = 1.f / sqrtf(ss / (float)len + eps);
+    for (int i = threadIdx.x; i < len; i += 256) hy_st(out + (size_t)t * ldo + i, row[i] * r * w[i]);
+}
+
+// z <- cap tanh(z / cap)
+static __global__ __launch_bounds__(256) void hy_softcap_kernel(float* __restrict__ z, size_t n, float cap) {
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) z[i] = cap * tanhf(z[i] / cap);
+}
+
+// Per-head products out[t][h][c] = sum_k in[t][h][k] Wt[h][k][c] (float32), optionally times sigmoid(gate[t][h][c]) (gate_mode 2:
+// sigmoid(gate[t][h]), one gate per head), for portions of a
 // few tokens (decode).  Two uses: the query carried into the latent's space, qa = Wk^T q (scores are then plain dot products with the
 // cached latents: q . (Wk c) = (Wk^T q) . c), and the value expansion applied after the weighted sum of latents.  Workgroup = (TT tokens, head, 64 columns): lane =
 // column, the four wavefronts split k and meet in LDS, a weight is read once for TT tokens.
 template <typename TO, int TT>
 static __global__ __launch_bounds__(256) void hy_headmm_kernel(const float* __restrict__ in, int ld_in, int K, int C, const float* __restrict__ Wt,
-                                                               const float* __restrict__ gate, int ldg, TO* __restrict__ out, int ldo, int n) {
+                                                               const float* __restrict__ gate, int ldg, TO* __restrict__ out, int ldo, int n, int gate_mode = 1) {
     __shared__ float red[3][TT][64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, h = blockIdx.y, c = blockIdx.z * 64 + lane, t0 = blockIdx.x * TT;
     const bool livec = c < C;
@@ -592,7 +654,7 @@ static __global__ __launch_bounds__(256) void hy_headmm_kernel(const float* __re
     for (int i = 0; i < TT; ++i) {
         if (t0 + i >= n) break;
         float v = (acc[i] + red[0][i][lane]) + (red[1][i][lane] + red[2][i][lane]);
-        if (gate) v *= hy_sigmoid(gate[(size_t)(t0 + i) * ldg + h * C + c]);
+        if (gate) v *= hy_sigmoid(gate[(size_t)(t0 + i) * ldg + (gate_mode == 2 ? h : h * C + c)]);
         hy_st(out + (size_t)(t0 + i) * ldo + h * C + c, v);
     }
 }
@@ -886,7 +948,8 @@ static __global__ __launch_bounds__(256) void hy_conv_tail_kernel(const float* _
 // Recurrence S_t = a_t S_(t-1) + b_t k_t x_t^T,  y_t = S_t^T q_t + D x_t  per head, S = N x P (keys / queries of N entries, values of P).
 // Three sources of a_t, b_t (HyScanArgs.mode): 0, a state-space layer: dt = softplus(raw + bias), a = e^(-e^(A_log) dt), b = dt, keys
 // and queries shared by the heads of a group; 1, gates that a kernel before this one left per (token, head) (hy_mem_gates_kernel);
-// 2, a fixed decay per head, b = 1.  Keys and queries are multiplied by k_mul / q_mul on the way into LDS and may turn there by their
+// 2, a fixed decay per head, b = 1.  Keys, queries and x may pass through silu on the way into LDS (act); keys and queries are
+// multiplied by k_mul / q_mul there and may turn by their
 // position (rot: first `dims` entries, pairs (i, i + dims / 2) or (2 i, 2 i + 1), angle = position * freq[i]).  ones_col: the last of
 // the P columns has x = 1 whatever the token (it then carries n_t = a n + b k, the normaliser of a matrix memory, and y's last column
 // is n_t . q_t).
@@ -902,6 +965,7 @@ struct HyScanArgs {
     const float* qsrc; int ldq, q_off, q_hstride;
     const float* xsrc; int ldx, x_off;                 // x of (t, head, column): xsrc + t ldx + x_off + head Px + column, Px = P - ones_col
     float k_mul, q_mul;
+    int act;                                           // 1: keys, queries and x are silu(source) (before the multipliers)
     HyScanRot rot;
     int mode;
     const float* dtsrc; int ld_dt, dt_off; const float* dt_bias; const float* A_log; const float* Dp;      // mode 0 (Dp: null = no skip term)
@@ -913,7 +977,7 @@ struct HyScanArgs {
     float* y; int ldy;                                 // y of (t, head, column): y + t ldy + head P + column
 };
 // rows t0 .. t0 + tb - 1 (N floats each, row stride ld) times mul -> dst[t Ns + n], zero behind N; eight loads in flight per thread
-__device__ __forceinline__ void hy_scan_stage(float* __restrict__ dst, const float* __restrict__ base, int ld, int t0, int tb, int N, int Ns, float mul) {
+__device__ __forceinline__ void hy_scan_stage(float* __restrict__ dst, const float* __restrict__ base, int ld, int t0, int tb, int N, int Ns, float mul, int act) {
     const int total = tb * Ns;
     for (int i0 = threadIdx.x; i0 < total; i0 += 8 * 256) {
         float v[8];
@@ -925,7 +989,7 @@ __device__ __forceinline__ void hy_scan_stage(float* __restrict__ dst, const flo
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
             const int i = i0 + u * 256;
-            if (i < total) dst[i] = v[u] * mul;
+            if (i < total) dst[i] = (act ? hy_silu(v[u]) : v[u]) * mul;
         }
     }
 }
@@ -973,11 +1037,12 @@ static __global__ __launch_bounds__(256) void hy_ssm_scan_kernel(HyScanArgs a) {
     for (int t0 = 0; t0 < n; t0 += TB) {
         const int tb = min(TB, n - t0);
         __syncthreads();
-        hy_scan_stage(sB, kbase, a.ldk, t0, tb, N, Ns, a.k_mul);
-        hy_scan_stage(sC, qbase, a.ldq, t0, tb, N, Ns, a.q_mul);
+        hy_scan_stage(sB, kbase, a.ldk, t0, tb, N, Ns, a.k_mul, a.act);
+        hy_scan_stage(sC, qbase, a.ldq, t0, tb, N, Ns, a.q_mul, a.act);
         for (int i = tid; i < tb * cols; i += 256) {
             const int t = i / cols, c = i - t * cols;
-            sX[i] = col0 + c < Px ? xbase[(size_t)(t0 + t) * a.ldx + col0 + c] : (col0 + c < P ? 1.f : 0.f);
+            if (col0 + c < Px) { const float xv = xbase[(size_t)(t0 + t) * a.ldx + col0 + c]; sX[i] = a.act ? hy_silu(xv) : xv; }
+            else sX[i] = col0 + c < P ? 1.f : 0.f;
         }
         if (tid < tb) {
             if (a.mode == 0) {

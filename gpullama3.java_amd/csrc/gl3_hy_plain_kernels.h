@@ -7,8 +7,9 @@
 
 // ---- residual update ----------------------------------------------------------------------------------------------------------------
 // One workgroup per token.  In this order, every part optional (null pointer = absent):
-//   x += ya_mul * ga * sum_z ya[z]              ya: a sublayer's output (or several sublayers' outputs), possibly as K-split parts; ga = sigmoid(gate_z[t * gate_ld]) or 1
-//   x += sum_k eo[pair_row[t top + k]]          the routed experts' down projections of this token
+//   d  = ya_mul * ga * sum_z ya[z]              ya: a sublayer's output (or several sublayers' outputs), possibly as K-split parts; ga = sigmoid(gate_z[t * gate_ld]) or 1
+//   d += sum_k ew[t top + k] eo[pair_row[t top + k]]   the routed experts' down projections of this token (ew: a weight per pair, null = 1)
+//   x += d, or with post_w: x += d / sqrt(mean(d^2) + eps) * post_w    (the sublayer's output passes a norm of its own before it joins the residual)
 //   x += yc / sqrt(mean(yc^2) + eps) * cw       a unit-RMS normed input with a plain weight
 //   hist_out[t] = x;  x = sum_j mix[j] hist[j][t], j < n_mix, where hist[n_mix - 1] is hist_out (what the layer leaves is an average over
 //                                               the embedding output and every layer's result so far)
@@ -17,7 +18,8 @@
 struct HyResid {
     float* x; int W;
     const float* ya; int ya_parts; size_t ya_stride; const float* gate_z; int gate_ld; float ya_mul;
-    const float* eo; const int* pair_row; int top;
+    const float* eo; const int* pair_row; int top; const float* ew;
+    const float* post_w;
     const float* yc; const float* cw;
     float* hist; size_t hist_stride; int n_mix; const float* mix;      // hist_out = hist + (n_mix - 1) hist_stride
     float* tap;
@@ -60,6 +62,34 @@ static __global__ __launch_bounds__(NT) void hy_resid_kernel(HyResid a, TO* __re
         cr = 1.f / sqrtf(ss / (float)W + a.eps);
     }
     const float ga = (a.gate_z ? hy_sigmoid(a.gate_z[(size_t)t * a.gate_ld]) : 1.f) * a.ya_mul;
+    float pr = 0.f;          // post_w: 1 / rms of the sublayer's whole output (the same sums as below, once more)
+    if (a.post_w) {
+        float sd = 0.f;
+        for (int w = threadIdx.x * V; w < W; w += NT * V) {
+            float y[V], e[V];
+#pragma unroll
+            for (int i = 0; i < V; ++i) y[i] = e[i] = 0.f;
+            if (a.ya)
+                for (int z = 0; z < a.ya_parts; ++z) {
+                    float q[V];
+                    hy_ldv<V>(a.ya + z * a.ya_stride + row + w, q);
+#pragma unroll
+                    for (int i = 0; i < V; ++i) y[i] += q[i];
+                }
+            if (a.eo)
+                for (int k = 0; k < a.top; ++k) {
+                    float q[V];
+                    hy_ldv<V>(a.eo + (size_t)a.pair_row[t * a.top + k] * W + w, q);
+                    const float wk = a.ew ? a.ew[t * a.top + k] : 1.f;
+#pragma unroll
+                    for (int i = 0; i < V; ++i) e[i] = fmaf(wk, q[i], e[i]);
+                }
+#pragma unroll
+            for (int i = 0; i < V; ++i) { const float d = ga * y[i] + e[i]; sd += d * d; }
+        }
+        sd = hy_block_sum<NT>(sd, red);
+        pr = 1.f / sqrtf(sd / (float)W + a.eps);
+    }
     float ss = 0.f, keep[HY_RC][V];
     int it = 0;
     for (int w = threadIdx.x * V; w < W; w += NT * V, ++it) {
@@ -88,16 +118,26 @@ static __global__ __launch_bounds__(NT) void hy_resid_kernel(HyResid a, TO* __re
             for (int k = 0; k < a.top; ++k) {
                 float q[V];
                 hy_ldv<V>(a.eo + (size_t)a.pair_row[t * a.top + k] * W + w, q);
+                const float wk = a.ew ? a.ew[t * a.top + k] : 1.f;
 #pragma unroll
-                for (int i = 0; i < V; ++i) e[i] += q[i];
+                for (int i = 0; i < V; ++i) e[i] = fmaf(wk, q[i], e[i]);
             }
         if (a.yc) { hy_ldv<V>(a.yc + row + w, c); hy_ldv<V>(a.cw + w, cw); }
+        if (a.post_w) {
+            float pw[V];
+            hy_ldv<V>(a.post_w + w, pw);
 #pragma unroll
-        for (int i = 0; i < V; ++i) {
-            x[i] += ga * y[i];
-            x[i] += e[i];
-            if (a.yc) x[i] += c[i] * cr * cw[i];
+            for (int i = 0; i < V; ++i) x[i] += (ga * y[i] + e[i]) * pr * pw[i];
+        } else {
+#pragma unroll
+            for (int i = 0; i < V; ++i) {
+                x[i] += ga * y[i];
+                x[i] += e[i];
+            }
         }
+#pragma unroll
+        for (int i = 0; i < V; ++i)
+            if (a.yc) x[i] += c[i] * cr * cw[i];
         if (a.hist) {
             hy_stv<V>(a.hist + (size_t)(a.n_mix - 1) * a.hist_stride + row + w, x);
             float m[V];
@@ -169,14 +209,20 @@ static __global__ __launch_bounds__(256) void hy_side_act_kernel(const float* __
 
 // ---- mixture of experts ---------------------------------------------------------------------------------------------------------------
 // Router: one wavefront per token.  z[t][0 .. E) are the router's float32 products (the sum of `parts` K-split partial products,
-// pstride apart); score = sigmoid(z); the `top` largest scores are taken in descending order (the lowest index wins a tie):
-// sel[t top + k], wgt[t top + k] = score.  E <= 64 * HY_RT_PER.  pair_row != null (a few tokens): the pairs keep their own order,
-// pair_row[p] = p.  extra_out != null: column E of z (the shared expert's gate logit) is summed into extra_out[t].
+// pstride apart); score = sigmoid(z), or softmax(z) over all E experts (HyRoute.softmax); the `top` largest of score (+ bias[e], where
+// bias != null: it decides the choice only) are taken in descending order (the lowest index wins a tie): sel[t top + k], wgt[t top + k] =
+// the chosen expert's score (without the bias), divided by the chosen scores' sum + 1e-20 (renorm), times mul.  E <= 64 * HY_RT_PER.
+// pair_row != null (a few tokens): the pairs keep their own order, pair_row[p] = p.  extra_out != null: column E of z (the shared
+// expert's gate logit) is summed into extra_out[t].
 constexpr int HY_RT_PER = 16;
+struct HyRoute { int softmax; const float* bias; int renorm; float mul; };
 static __global__ __launch_bounds__(64) void hy_route_kernel(const float* __restrict__ z, int ldz, int parts, size_t pstride, int E, int top, int* __restrict__ sel,
-                                                             float* __restrict__ wgt, int* __restrict__ pair_row, float* __restrict__ extra_out) {
+                                                             float* __restrict__ wgt, int* __restrict__ pair_row, float* __restrict__ extra_out,
+                                                             HyRoute rt = HyRoute{0, nullptr, 0, 1.f}) {
     const int t = blockIdx.x, lane = threadIdx.x;
-    float s[HY_RT_PER];
+    constexpr float GONE = -3.0e38f;
+    float s[HY_RT_PER], c[HY_RT_PER];          // score; what the choice goes by
+    float zmax = -INFINITY;
 #pragma unroll
     for (int i = 0; i < HY_RT_PER; ++i) {
         const int e = lane + 64 * i;
@@ -184,27 +230,51 @@ static __global__ __launch_bounds__(64) void hy_route_kernel(const float* __rest
         if (e < E + (extra_out ? 1 : 0))
             for (int p = 0; p < parts; ++p) v += z[p * pstride + (size_t)t * ldz + e];
         if (extra_out && e == E) extra_out[t] = v;
-        s[i] = e < E ? hy_sigmoid(v) : -1.f;
+        s[i] = v;
+        if (e < E) zmax = fmaxf(zmax, v);
     }
+    if (rt.softmax) {
+        zmax = hy_wave_max(zmax);
+        float den = 0.f;
+#pragma unroll
+        for (int i = 0; i < HY_RT_PER; ++i) { s[i] = lane + 64 * i < E ? expf(s[i] - zmax) : 0.f; den += s[i]; }
+        den = hy_wave_sum(den);
+#pragma unroll
+        for (int i = 0; i < HY_RT_PER; ++i) s[i] = s[i] / den;
+    } else {
+#pragma unroll
+        for (int i = 0; i < HY_RT_PER; ++i) s[i] = hy_sigmoid(s[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < HY_RT_PER; ++i) {
+        const int e = lane + 64 * i;
+        c[i] = e < E ? s[i] + (rt.bias ? rt.bias[e] : 0.f) : GONE;
+    }
+    float wsum = 0.f;
     for (int k = 0; k < top; ++k) {
-        float best = -2.f;
+        float best = GONE, bs = 0.f;
         int bi = 0x7fffffff;
 #pragma unroll
         for (int i = 0; i < HY_RT_PER; ++i)
-            if (s[i] > best) { best = s[i]; bi = lane + 64 * i; }        // ascending index within a lane: strict > keeps the lowest
+            if (c[i] > best) { best = c[i]; bs = s[i]; bi = lane + 64 * i; }        // ascending index within a lane: strict > keeps the lowest
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) {
-            const float ob = __shfl_xor(best, o, 64);
+            const float ob = __shfl_xor(best, o, 64), os = __shfl_xor(bs, o, 64);
             const int oi = __shfl_xor(bi, o, 64);
-            if (ob > best || (ob == best && oi < bi)) { best = ob; bi = oi; }
+            if (ob > best || (ob == best && oi < bi)) { best = ob; bs = os; bi = oi; }
         }
+        wsum += bs;
         if (lane == 0) {
-            sel[t * top + k] = bi; wgt[t * top + k] = best;
+            sel[t * top + k] = bi; wgt[t * top + k] = bs;
             if (pair_row) pair_row[t * top + k] = t * top + k;
         }
 #pragma unroll
         for (int i = 0; i < HY_RT_PER; ++i)
-            if (lane + 64 * i == bi) s[i] = -1.f;
+            if (lane + 64 * i == bi) c[i] = GONE;
+    }
+    if (lane == 0 && (rt.renorm || rt.mul != 1.f)) {          // the lane rereads what it wrote
+        const float m = rt.mul / (rt.renorm ? wsum + 1e-20f : 1.f);
+        for (int k = 0; k < top; ++k) wgt[t * top + k] *= m;
     }
 }
 
@@ -235,12 +305,12 @@ static __global__ __launch_bounds__(256) void hy_moe_group_kernel(const int* __r
     __syncthreads();
     for (int p = threadIdx.x; p < P; p += 256) pair_row[p] = atomicAdd(&cnt[sel[p]], 1);
 }
-// The experts' operand: row pair_row[p] = wgt[p] * h[token of p] (a score scales its expert's INPUT), in the matrix type.
+// The experts' operand: row pair_row[p] = wgt[p] * h[token of p] (a score scales its expert's INPUT; wgt = null: the plain row), in the matrix type.
 template <typename T>
 static __global__ __launch_bounds__(256) void hy_moe_scale_kernel(const T* __restrict__ h, int W, int top, const float* __restrict__ wgt, const int* __restrict__ pair_row,
                                                                   T* __restrict__ out) {
     const int p = blockIdx.x, t = p / top;
-    const float s = wgt[p];
+    const float s = wgt ? wgt[p] : 1.f;
     T* dst = out + (size_t)pair_row[p] * W;
     for (int w = threadIdx.x; w < W; w += 256) hy_st(dst + w, s * hy_ld(h + (size_t)t * W + w));
 }

@@ -46,7 +46,16 @@ struct HyLayer {
     float* hc[2][3] = {};      // per sublayer: in [S], out [S], mix [S x S]
     // latent: norm weight; key expansion [H D][R] (as stored: rows for the expansion GEMM, and [h][d][r] for carrying a query into the latent's
     // space); value expansion as stored [H V][R] (GEMM) and transposed [H][R][V] (expansion of a weighted sum of latents)
+    // With a rotated part (rot_dim > 0) the cached row is [latent | turned key part] (Re = kv_rank + rot_dim entries) and a query head has
+    // De = dim + rot_dim entries; the expansions are padded to these sizes (key expansion: identity behind the latent's columns, value
+    // expansion: zeros), so every kernel of the latent path runs on (De, Re) as it does on (dim, kv_rank) without a rotated part.
     float *lat_norm = nullptr, *wk = nullptr, *wv = nullptr, *wvT = nullptr;
+    int De = 0, Re = 0;
+    HyMat uq;                  // latent with q_rank: query expansion [heads De x q_rank]
+    float* qlat_norm = nullptr;// norm weight of the query latent [q_rank]
+    float rot_mscale = 1.f;    // multiplier of cos and sin (YaRN)
+    float *norm1b = nullptr, *norm2b = nullptr;      // post norms of the two sublayers
+    float* route_bias = nullptr;                     // mixture of experts: added to the scores for the choice
     float *conv_w = nullptr, *conv_b = nullptr, *dt_bias = nullptr, *a_log = nullptr, *dskip = nullptr, *ssm_norm = nullptr;
     size_t off_k = 0, off_v = 0, off_state = 0, off_tail = 0;       // float offsets inside a sequence slot
     uint64_t have = 0;
@@ -61,6 +70,10 @@ struct gl3_hybrid_state {
     float emb_scale = 1.f, norm_offset = 0.f;
     int side_dim = 0, side_ld = 0, max_top = 0;
     bool depth = false;
+    bool post_norms = false;   // every sublayer's output passes an RMS norm with its own weight before it joins the residual
+    float softcap = 0.f;       // logits <- cap tanh(logits / cap); 0 = none
+    void* cq = nullptr;        // latent with q_rank: the normed query latents [mb][max q_rank], matrix type
+    float* qfull = nullptr;    // ... and the expanded queries [mb][max heads De]
     HyMat side_emb;            // [vocab][layers * side_dim]
     // [layers + 1][mb][W]; K-split parts of [mb][side_dim] and of [mb][experts + 1]; the shared expert's gate logit [mb]; [mb top]; [mb top][W]
     float *hist = nullptr, *side_z = nullptr, *moe_z = nullptr, *sgz = nullptr, *wsel = nullptr, *eout = nullptr;

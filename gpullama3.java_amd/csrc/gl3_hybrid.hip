@@ -58,7 +58,7 @@ static int hy_gate_rows(const gl3_layer_desc& d) { return d.mixer == GL3_MIX_MEM
 static int hy_proj_rows(const gl3_layer_desc& d) {
     switch (d.mixer) {
         case GL3_MIX_ATTENTION: return d.heads * d.dim + d.kv_heads * d.dim + d.kv_heads * d.vdim + hy_gate_rows(d);
-        case GL3_MIX_LATENT: return d.heads * d.dim + d.kv_rank + hy_gate_rows(d);
+        case GL3_MIX_LATENT: return (d.q_rank > 0 ? d.q_rank : d.heads * (d.dim + d.rot_dim)) + (d.kv_share > 0 ? 0 : d.kv_rank + d.rot_dim) + hy_gate_rows(d);
         case GL3_MIX_MEMORY: return 2 * d.heads * d.dim + 2 * d.heads * d.vdim + (d.mem_gates == GL3_MEM_EXP_GATES ? 2 * d.heads : 0);
         default: return 2 * d.heads * d.vdim + 2 * d.groups * d.state + d.heads;
     }
@@ -74,6 +74,7 @@ static const char* hy_check_layer(const gl3_layer_desc& d) {
     if (d.experts < 0 || d.shared_ff < 0) return "experts and shared_ff must be >= 0";
     if (d.experts > 0) {
         if (d.ff < 1) return "mixture of experts: ff (one expert's width) must be positive";
+        if (d.ff_act == 2) return "mixture of experts: the experts are gated (ff_act 0 or 1)";
         if (d.experts + (d.shared_ff > 0 ? 1 : 0) > 64 * HY_RT_PER) return "mixture of experts: at most 1024 router rows (experts, plus one for a shared expert's gate)";
         if (d.top < 1 || d.top > d.experts || d.top > 64) return "mixture of experts: 1 <= top <= min(experts, 64)";
     } else if (d.shared_ff > 0)
@@ -81,7 +82,9 @@ static const char* hy_check_layer(const gl3_layer_desc& d) {
     if (d.mixer != GL3_MIX_ATTENTION && (d.v_unit_norm || d.v_rot || d.window > 0 || d.keep_first > 0 || d.pool > 0 || d.qk_bias))
         return "value norm / rotation, windows, pooled blocks and q / k / v biases belong to the attention mixer";
     if (d.mixer != GL3_MIX_ATTENTION && d.mixer != GL3_MIX_MEMORY && d.rot_dims) return "rotary positions belong to the attention and matrix-memory mixers";
-    if (d.ff_act < 0 || d.ff_act > 1) return "ff_act must be 0 or 1";
+    if (d.ff_act < 0 || d.ff_act > 2) return "ff_act must be 0, 1 or 2";
+    if (d.mixer != GL3_MIX_LATENT && (d.q_rank || d.rot_dim || d.kv_share)) return "q_rank, rot_dim and kv_share belong to the latent attention";
+    if (d.mixer != GL3_MIX_MEMORY && (d.mem_qkv_act || d.mem_norm_whole)) return "mem_qkv_act and mem_norm_whole belong to the matrix memory";
     if (d.mixer == GL3_MIX_ATTENTION) {
         if (d.kv_heads < 1 || d.heads % d.kv_heads) return "attention: heads must be a multiple of kv_heads";
         if (d.dim < 1) return "attention: dim must be positive";
@@ -95,7 +98,12 @@ static const char* hy_check_layer(const gl3_layer_desc& d) {
         if (d.pool > 0 && d.slope_log2 != 0.f) return "attention: pooled blocks have no distance term";
     } else if (d.mixer == GL3_MIX_LATENT) {
         if (d.dim < 1 || d.kv_rank < 1) return "latent attention: dim and kv_rank must be positive";
-        if (d.kv_rank > 512) return "latent attention: kv_rank <= 512";
+        if (d.rot_dim < 0 || (d.rot_dim & 1)) return "latent attention: rot_dim must be even and >= 0";
+        if (d.kv_rank + d.rot_dim > 512) return "latent attention: kv_rank + rot_dim <= 512";
+        if (d.rot_dim > 0 && !(d.rot_base > 0.f)) return "latent attention: rot_base must be positive";
+        if (d.rot_dim > 0 && d.rot_yarn_factor > 0.f && !(d.rot_yarn_original > 0.f && d.rot_yarn_fast > 0.f && d.rot_yarn_slow > 0.f && d.rot_base != 1.f))
+            return "latent attention: scaled frequencies need original, fast and slow > 0";
+        if (d.q_rank < 0 || d.kv_share < 0) return "latent attention: q_rank and kv_share must be >= 0";
     } else if (d.mixer == GL3_MIX_MEMORY) {
         if (d.dim < 1 || d.dim > 2048) return "matrix memory: 1 <= dim <= 2048";
         if (d.rot_dims < 0 || d.rot_dims > d.dim || (d.rot_dims & 1)) return "matrix memory: rot_dims must be even and at most dim";
@@ -123,11 +131,20 @@ int32_t gl3_hy_create(const gl3_model_desc* desc, gl3_ctx** out, std::string& er
     if (desc->dim < 1 || desc->vocab < 1 || desc->ctx < 1) { err = "layer-list family: dim, vocab and ctx must be positive"; return GL3_E_ARG; }
     if (desc->weight_type != GL3_TYPE_BF16 && desc->weight_type != GL3_TYPE_F32) { err = "layer-list family: weight_type must be GL3_TYPE_BF16 (or GL3_TYPE_F32)"; return GL3_E_UNSUPPORTED; }
     if (desc->tp_size > 1) { err = "layer-list family: tensor parallelism is not built"; return GL3_E_UNSUPPORTED; }
+    if (desc->post_norms && (desc->streams > 0 || desc->side_dim || desc->depth_mix || desc->parallel_block)) { err = "layer-list family: post norms need the plain residual without token input, depth average and parallel block"; return GL3_E_ARG; }
+    if (desc->logit_softcap < 0.f) { err = "layer-list family: logit_softcap must be >= 0"; return GL3_E_ARG; }
     if (desc->parallel_block && (desc->streams > 0 || desc->side_dim || desc->depth_mix)) { err = "layer-list family: the parallel block needs the plain residual without token input and depth average"; return GL3_E_ARG; }
     for (int l = 0; l < desc->n_layers; ++l) {
         const gl3_layer_desc& ld = desc->layer_descs[l];
         if (const char* m = hy_check_layer(ld)) { err = "layer " + std::to_string(l) + ": " + m; return GL3_E_ARG; }
         if (desc->parallel_block && ld.experts > 0) { err = "layer-list family: the parallel block has a dense feed-forward"; return GL3_E_ARG; }
+        if (ld.mixer == GL3_MIX_LATENT && ld.kv_share > 0) {          // the cache it reads: an earlier latent layer with rows of its own and the same row layout
+            const int j = ld.kv_share - 1;
+            const gl3_layer_desc* o = j < l ? &desc->layer_descs[j] : nullptr;
+            if (!o || o->mixer != GL3_MIX_LATENT || o->kv_share > 0 || o->kv_rank != ld.kv_rank || o->rot_dim != ld.rot_dim) {
+                err = "layer " + std::to_string(l) + ": kv_share must name an earlier latent-attention layer with a cache of its own and the same kv_rank and rot_dim"; return GL3_E_ARG;
+            }
+        }
         if (ld.beside) {
             if (ld.beside->mixer == GL3_MIX_LATENT || ld.mixer == GL3_MIX_LATENT || ld.beside->mixer == GL3_MIX_SSM || ld.mixer == GL3_MIX_SSM) {
                 err = "layer " + std::to_string(l) + ": only attention and matrix-memory mixers can stand side by side"; return GL3_E_ARG;
@@ -149,6 +166,8 @@ int32_t gl3_hy_create(const gl3_model_desc* desc, gl3_ctx** out, std::string& er
     h->norm_offset = desc->norm_offset;
     h->side_dim = desc->side_dim; h->side_ld = hy_cdiv(std::max(1, desc->side_dim), 8) * 8;
     h->depth = desc->depth_mix != 0;
+    h->post_norms = desc->post_norms != 0;
+    h->softcap = desc->logit_softcap;
     h->S = std::max(1, desc->streams); h->W = desc->dim; h->mb = std::max(1, desc->max_batch); h->n_seqs = ctx->n_seqs;
     h->want_cap = std::min(h->mb, 256);
     h->busy.assign(h->n_seqs, 0); h->len.assign(h->n_seqs, 0);
@@ -167,7 +186,7 @@ int32_t gl3_hy_create(const gl3_model_desc* desc, gl3_ctx** out, std::string& er
     size_t slot = 0;
     int max_proj = 1, max_mix = W, max_ch = 1, max_inner = 1, max_hr = 1, max_hdv = 1, max_kx = 0, max_vx = 0, max_rz = 0, max_top = 0, max_eff = 0, max_e = 0;
     if (h->side_dim > 0) TRY(hy_alloc_mat(ctx, h->side_emb, V, desc->n_layers * h->side_dim, desc->n_layers * h->side_dim));
-    int max_heads = 1;
+    int max_heads = 1, max_qr = 0, max_qfull = 0;
     // one mixer's share of the layer: its offsets in the fused projection row (p0 = its first row) and in mixo / o (o0 = its first
     // column), its vectors and tables, its part of the sequence slot
     auto setup_mixer = [&](HyLayer& Ly, int p0, int o0) -> int32_t {
@@ -201,14 +220,44 @@ int32_t gl3_hy_create(const gl3_model_desc* desc, gl3_ctx** out, std::string& er
             if (d.softmax_sink == 2) TRYM(hy_alloc(ctx, &Ly.sink, (size_t)d.heads * 4));
             max_hdv = std::max(max_hdv, d.heads * d.vdim);
         } else if (d.mixer == GL3_MIX_LATENT) {
-            Ly.q_off = p0; Ly.c_off = Ly.q_off + d.heads * d.dim; Ly.g_off = Ly.c_off + d.kv_rank;
-            Ly.off_k = Ly.off_v = slot; slot += (size_t)C * d.kv_rank;
-            TRYM(hy_alloc(ctx, &Ly.lat_norm, (size_t)d.kv_rank * 4));
-            TRYM(hy_alloc(ctx, &Ly.wk, (size_t)d.heads * d.dim * d.kv_rank * 4));
-            TRYM(hy_alloc(ctx, &Ly.wv, (size_t)d.heads * d.vdim * d.kv_rank * 4));
-            TRYM(hy_alloc(ctx, &Ly.wvT, (size_t)d.heads * d.vdim * d.kv_rank * 4));
-            max_hr = std::max(max_hr, d.heads * d.kv_rank); max_hdv = std::max(max_hdv, std::max(d.heads * d.kv_rank, d.heads * d.vdim));
-            max_kx = std::max(max_kx, d.heads * d.dim); max_vx = std::max(max_vx, d.heads * d.vdim);
+            const int De = Ly.De = d.dim + d.rot_dim, Re = Ly.Re = d.kv_rank + d.rot_dim;
+            Ly.q_off = p0; Ly.c_off = Ly.q_off + (d.q_rank > 0 ? d.q_rank : d.heads * De); Ly.g_off = Ly.c_off + (d.kv_share > 0 ? 0 : Re);
+            if (d.kv_share > 0) Ly.off_k = Ly.off_v = h->L[d.kv_share - 1].off_k;          // another layer's rows
+            else {
+                Ly.off_k = Ly.off_v = slot; slot += (size_t)C * Re;
+                TRYM(hy_alloc(ctx, &Ly.lat_norm, (size_t)d.kv_rank * 4));
+            }
+            TRYM(hy_alloc(ctx, &Ly.wk, (size_t)d.heads * De * Re * 4));
+            TRYM(hy_alloc(ctx, &Ly.wv, (size_t)d.heads * d.vdim * Re * 4));
+            TRYM(hy_alloc(ctx, &Ly.wvT, (size_t)d.heads * d.vdim * Re * 4));
+            if (d.q_rank > 0) {
+                TRYM(hy_alloc_mat(ctx, Ly.uq, d.heads * De, d.q_rank, d.q_rank));
+                TRYM(hy_alloc(ctx, &Ly.qlat_norm, (size_t)d.q_rank * 4));
+                max_qr = std::max(max_qr, d.q_rank); max_qfull = std::max(max_qfull, d.heads * De);
+            }
+            if (d.rot_dim > 0) {
+                // frequencies of the rotated part, made in double: base^(-2 i / n), blended with the / factor frequency along a ramp over the
+                // pair index when rot_yarn_factor > 0; cos and sin then carry the multiplier 0.1 ln(factor) + 1
+                const int n = d.rot_dim;
+                std::vector<float> f(n / 2);
+                const double base = d.rot_base, factor = d.rot_yarn_factor;
+                double lo = 0, hi = 0;
+                if (factor > 0.0) {
+                    auto where = [&](double turns) { return n * std::log((double)d.rot_yarn_original / (2.0 * M_PI * turns)) / (2.0 * std::log(base)); };
+                    lo = std::max(std::floor(where(d.rot_yarn_fast)), 0.0);
+                    hi = std::min(std::ceil(where(d.rot_yarn_slow)), (double)(n - 1));
+                    Ly.rot_mscale = (float)(0.1 * std::log(factor) + 1.0);
+                }
+                for (int i = 0; i < n / 2; ++i) {
+                    const double fi = std::pow(base, -2.0 * i / n);
+                    const double ramp = factor > 0.0 ? std::min(1.0, std::max(0.0, (i - lo) / std::max(hi - lo, 0.001))) : 0.0;
+                    f[i] = (float)(factor > 0.0 ? fi / factor * ramp + fi * (1.0 - ramp) : fi);
+                }
+                TRYM(hy_alloc(ctx, &Ly.rot_freq, f.size() * 4));
+                if (hipMemcpy(Ly.rot_freq, f.data(), f.size() * 4, hipMemcpyHostToDevice) != hipSuccess) { ctx->err = "copy of the rotary table failed"; return GL3_E_HIP; }
+            }
+            max_hr = std::max(max_hr, d.heads * Re); max_hdv = std::max(max_hdv, std::max(d.heads * Re, d.heads * d.vdim));
+            max_kx = std::max(max_kx, d.heads * De); max_vx = std::max(max_vx, d.heads * d.vdim);
         } else if (d.mixer == GL3_MIX_MEMORY) {
             const bool eg = d.mem_gates == GL3_MEM_EXP_GATES;
             Ly.d.kv_heads = d.heads;
@@ -272,15 +321,20 @@ int32_t gl3_hy_create(const gl3_model_desc* desc, gl3_ctx** out, std::string& er
         Ly.dense_ff = d.experts > 0 ? d.shared_ff : d.ff;
         Ly.dense_limit = d.experts > 0 ? d.shared_limit : d.ff_limit;
         if (d.ff > 0 && !h->parallel) TRY(hy_alloc(ctx, &Ly.norm2, (size_t)W * 4));
+        if (h->post_norms) {
+            TRY(hy_alloc(ctx, &Ly.norm1b, (size_t)W * 4));
+            if (d.ff > 0) TRY(hy_alloc(ctx, &Ly.norm2b, (size_t)W * 4));
+        }
         if (Ly.dense_ff > 0) {
             Ly.ff_pad = hy_cdiv(Ly.dense_ff, 32) * 32;
-            TRY(hy_alloc_mat(ctx, Ly.gu, 2 * Ly.ff_pad, W, W));
+            TRY(hy_alloc_mat(ctx, Ly.gu, (d.experts == 0 && d.ff_act == 2 ? 1 : 2) * Ly.ff_pad, W, W));          // without a gate: the up rows alone
             TRY(hy_alloc_mat(ctx, Ly.down, W, Ly.ff_pad, Ly.ff_pad));
             max_mix = std::max(max_mix, Ly.ff_pad);
         }
         if (d.experts > 0) {
             Ly.eff_pad = hy_cdiv(d.ff, 32) * 32;
-            TRY(hy_alloc_mat(ctx, Ly.router, d.experts + (d.shared_ff > 0 ? 1 : 0), W, W));
+            TRY(hy_alloc_mat(ctx, Ly.router, d.experts + (d.shared_ff > 0 && !d.shared_ungated ? 1 : 0), W, W));
+            if (d.route_bias) TRY(hy_alloc(ctx, &Ly.route_bias, (size_t)d.experts * 4));
             TRY(hy_alloc_mat(ctx, Ly.egu, d.experts * 2 * Ly.eff_pad, W, W));
             TRY(hy_alloc_mat(ctx, Ly.edown, d.experts * W, Ly.eff_pad, Ly.eff_pad));
             max_rz = std::max(max_rz, Ly.router.rows); max_top = std::max(max_top, d.top); max_eff = std::max(max_eff, Ly.eff_pad); max_e = std::max(max_e, d.experts);
@@ -307,6 +361,10 @@ int32_t gl3_hy_create(const gl3_model_desc* desc, gl3_ctx** out, std::string& er
     TRY(hy_alloc(ctx, &h->ssm_y, (size_t)mb * max_inner * 4));
     TRY(hy_alloc(ctx, &h->qa, (size_t)mb * max_hr * 4));
     TRY(hy_alloc(ctx, &h->oc, (size_t)mb * max_hr * 4));
+    if (max_qr > 0) {
+        TRY(hy_alloc(ctx, &h->cq, (size_t)mb * max_qr * es));
+        TRY(hy_alloc(ctx, &h->qfull, (size_t)mb * max_qfull * 4));
+    }
     if (max_kx > 0 && mb > 8) {          // latent attention, portions of many tokens: expanded keys / values of one layer at a time
         TRY(hy_alloc(ctx, &h->kx, (size_t)C * max_kx * 4));
         TRY(hy_alloc(ctx, &h->vx, (size_t)C * max_vx * 4));
@@ -379,14 +437,16 @@ void gl3_hy_destroy(gl3_ctx* ctx) {
         for (HyLayer* M : {&L, L.side}) {
             if (!M) continue;
             f(M->lat_norm); f(M->wk); f(M->wv); f(M->wvT); f(M->conv_w); f(M->conv_b); f(M->dt_bias); f(M->a_log); f(M->dskip); f(M->ssm_norm);
-            f(M->rot_freq); f(M->vrot_freq); f(M->qn); f(M->kn); f(M->sink); f(M->decay);
+            f(M->rot_freq); f(M->vrot_freq); f(M->qn); f(M->kn); f(M->sink); f(M->decay); f(M->uq.w); f(M->qlat_norm);
         }
         delete L.side;
         L.side = nullptr;
+        f(L.norm1b); f(L.norm2b); f(L.route_bias);
         f(L.router.w); f(L.egu.w); f(L.edown.w); f(L.depth_mix); f(L.side_gate.w); f(L.side_proj.w); f(L.side_norm);
     }
     f(h->side_emb.w); f(h->sgz); f(h->hist); f(h->side_z); f(h->moe_z); f(h->wsel); f(h->eout); f(h->xb); f(h->side_g); f(h->ea); f(h->eact); f(h->sel); f(h->pair_row); f(h->tiles); f(h->ntiles);
     f(h->slots); f(h->X); f(h->h); f(h->proj); f(h->y); f(h->mixo); f(h->conv); f(h->ssm_y); f(h->qa); f(h->oc); f(h->kx); f(h->vx); f(h->part_acc); f(h->part_ml); f(h->gates); f(h->rowr);
+    f(h->cq); f(h->qfull);
     f(h->xw); f(h->logits); f(h->taps); f(h->ones); f(h->dyn);
     hf(h->h_dyn); hf(h->h_logits);
     if (ctx->logits == h->logits) ctx->logits = nullptr;
@@ -477,7 +537,16 @@ int32_t gl3_hy_upload(gl3_ctx* ctx, int32_t id, int32_t layer, const void* host,
     switch (id) {
         case GL3_T_ATTN_NORM: if (!beside) r = hy_put_vec(ctx, L.norm1, W, host, bytes, type, h->norm_offset); break;
         case GL3_T_FFN_NORM: if (d.ff > 0 && L.norm2) r = hy_put_vec(ctx, L.norm2, W, host, bytes, type, h->norm_offset); break;
-        case GL3_T_WQ: if (att || lat || mem) r = hy_put_rows(ctx, proj, L.q_off, d.heads * d.dim, W, host, bytes, type, 0); break;
+        case GL3_T_ATTN_POST_NORM: if (!beside && L.norm1b) r = hy_put_vec(ctx, L.norm1b, W, host, bytes, type, h->norm_offset); break;
+        case GL3_T_FFN_POST_NORM: if (!beside && L.norm2b) r = hy_put_vec(ctx, L.norm2b, W, host, bytes, type, h->norm_offset); break;
+        case GL3_T_WQ:
+            if (lat && d.q_rank > 0) r = hy_put_rows(ctx, L.uq, 0, d.heads * L.De, d.q_rank, host, bytes, type, 0);
+            else if (lat) r = hy_put_rows(ctx, proj, L.q_off, d.heads * L.De, W, host, bytes, type, 0);
+            else if (att || mem) r = hy_put_rows(ctx, proj, L.q_off, d.heads * d.dim, W, host, bytes, type, 0);
+            break;
+        case GL3_T_Q_DOWN: if (lat && d.q_rank > 0) r = hy_put_rows(ctx, proj, L.q_off, d.q_rank, W, host, bytes, type, 0); break;
+        case GL3_T_Q_DOWN_NORM: if (lat && d.q_rank > 0) r = hy_put_vec(ctx, L.qlat_norm, d.q_rank, host, bytes, type); break;
+        case GL3_T_FFN_ROUTE_BIAS: if (d.experts > 0 && d.route_bias) r = hy_put_vec(ctx, L.route_bias, d.experts, host, bytes, type); break;
         case GL3_T_WK: if (att || mem) r = hy_put_rows(ctx, proj, L.k_off, d.kv_heads * d.dim, W, host, bytes, type, 0); break;
         case GL3_T_WV: if (att || mem) r = hy_put_rows(ctx, proj, L.v_off, d.kv_heads * d.vdim, W, host, bytes, type, 0); break;
         case GL3_T_ATTN_GATE: if (((att || lat) && d.out_gate) || mem) r = hy_put_rows(ctx, proj, L.g_off, hy_gate_rows(d), W, host, bytes, type, 0); break;
@@ -492,19 +561,36 @@ int32_t gl3_hy_upload(gl3_ctx* ctx, int32_t id, int32_t layer, const void* host,
         case GL3_T_MEM_FGATE: if (memg) r = hy_put_rows(ctx, proj, L.f_off, d.heads, W, host, bytes, type, 0); break;
         case GL3_T_MEM_IGATE_BIAS: if (memg) r = hy_put_vec(ctx, L.pbias + L.i_off, d.heads, host, bytes, type); break;
         case GL3_T_MEM_FGATE_BIAS: if (memg) r = hy_put_vec(ctx, L.pbias + L.f_off, d.heads, host, bytes, type); break;
-        case GL3_T_KV_DOWN: if (lat) r = hy_put_rows(ctx, proj, L.c_off, d.kv_rank, W, host, bytes, type, 0); break;
-        case GL3_T_KV_DOWN_NORM: if (lat) r = hy_put_vec(ctx, L.lat_norm, d.kv_rank, host, bytes, type); break;
-        case GL3_T_K_UP: if (lat) r = hy_put_vec(ctx, L.wk, (size_t)d.heads * d.dim * d.kv_rank, host, bytes, type); break;
+        case GL3_T_KV_DOWN: if (lat && d.kv_share == 0) r = hy_put_rows(ctx, proj, L.c_off, L.Re, W, host, bytes, type, 0); break;
+        case GL3_T_KV_DOWN_NORM: if (lat && d.kv_share == 0) r = hy_put_vec(ctx, L.lat_norm, d.kv_rank, host, bytes, type); break;
+        case GL3_T_K_UP:
+            if (lat) {          // [h][dim][kv_rank] -> [h][De][Re]: zeros behind the latent's columns, and the rotated entries pass (identity)
+                const int R = d.kv_rank, De = L.De, Re = L.Re;
+                if (!hy_to_f32(host, bytes, type, (size_t)d.heads * d.dim * R, f)) GL3_FAIL(GL3_E_ARG, "tensor size or type mismatch");
+                std::vector<float> wk((size_t)d.heads * De * Re, 0.f);
+                for (int hh = 0; hh < d.heads; ++hh) {
+                    for (int dd = 0; dd < d.dim; ++dd) memcpy(&wk[((size_t)hh * De + dd) * Re], &f[((size_t)hh * d.dim + dd) * R], (size_t)R * 4);
+                    for (int j = 0; j < d.rot_dim; ++j) wk[((size_t)hh * De + d.dim + j) * Re + R + j] = 1.f;
+                }
+                HY_HIP(hipMemcpy(L.wk, wk.data(), wk.size() * 4, hipMemcpyHostToDevice));
+                r = GL3_OK;
+            }
+            break;
         case GL3_T_V_UP:
-            if (lat) {
-                const size_t n = (size_t)d.heads * d.vdim * d.kv_rank;
-                if (!hy_to_f32(host, bytes, type, n, f)) GL3_FAIL(GL3_E_ARG, "tensor size or type mismatch");
-                std::vector<float> tr(n);                   // [h][v][r] -> [h][r][v]
+            if (lat) {          // [h][v][kv_rank] -> [h][v][Re] (zeros behind the latent's columns) and its transpose [h][Re][v]
+                const int R = d.kv_rank, Re = L.Re;
+                const size_t n = (size_t)d.heads * d.vdim * Re;
+                if (!hy_to_f32(host, bytes, type, (size_t)d.heads * d.vdim * R, f)) GL3_FAIL(GL3_E_ARG, "tensor size or type mismatch");
+                std::vector<float> wv(n, 0.f), tr(n, 0.f);
                 for (int hh = 0; hh < d.heads; ++hh)
                     for (int v = 0; v < d.vdim; ++v)
-                        for (int rr = 0; rr < d.kv_rank; ++rr) tr[((size_t)hh * d.kv_rank + rr) * d.vdim + v] = f[((size_t)hh * d.vdim + v) * d.kv_rank + rr];
+                        for (int rr = 0; rr < R; ++rr) {
+                            const float x = f[((size_t)hh * d.vdim + v) * R + rr];
+                            wv[((size_t)hh * d.vdim + v) * Re + rr] = x;
+                            tr[((size_t)hh * Re + rr) * d.vdim + v] = x;
+                        }
                 HY_HIP(hipMemcpy(L.wvT, tr.data(), n * 4, hipMemcpyHostToDevice));
-                HY_HIP(hipMemcpy(L.wv, f.data(), n * 4, hipMemcpyHostToDevice));
+                HY_HIP(hipMemcpy(L.wv, wv.data(), n * 4, hipMemcpyHostToDevice));
                 r = GL3_OK;
             }
             break;
@@ -515,8 +601,8 @@ int32_t gl3_hy_upload(gl3_ctx* ctx, int32_t id, int32_t layer, const void* host,
         case GL3_T_SSM_A_LOG: if (ssm) r = hy_put_vec(ctx, L.a_log, d.heads, host, bytes, type); break;
         case GL3_T_SSM_D: if (ssm) r = hy_put_vec(ctx, L.dskip, d.heads, host, bytes, type); break;
         case GL3_T_SSM_NORM: if (ssm || (mem && d.mem_norm_weight)) r = hy_put_vec(ctx, L.ssm_norm, mo, host, bytes, type); break;
-        case GL3_T_W1: if (L.dense_ff > 0) r = hy_put_rows(ctx, L.gu, 0, L.dense_ff, W, host, bytes, type, 1); break;
-        case GL3_T_W3: if (L.dense_ff > 0) r = hy_put_rows(ctx, L.gu, 0, L.dense_ff, W, host, bytes, type, 2); break;
+        case GL3_T_W1: if (L.dense_ff > 0 && (d.experts > 0 || d.ff_act != 2)) r = hy_put_rows(ctx, L.gu, 0, L.dense_ff, W, host, bytes, type, 1); break;
+        case GL3_T_W3: if (L.dense_ff > 0) r = hy_put_rows(ctx, L.gu, 0, L.dense_ff, W, host, bytes, type, (d.experts == 0 && d.ff_act == 2) ? 0 : 2); break;
         case GL3_T_W2:
             if (L.dense_ff > 0) {          // [W][ff] into rows of ff_pad
                 if (!hy_to_f32(host, bytes, type, (size_t)W * L.dense_ff, f)) GL3_FAIL(GL3_E_ARG, "tensor size or type mismatch");
@@ -527,7 +613,7 @@ int32_t gl3_hy_upload(gl3_ctx* ctx, int32_t id, int32_t layer, const void* host,
             break;
         // mixture of experts: router rows, then (one more row) the shared expert's gate; the experts' matrices arrive stacked [experts][..]
         case GL3_T_FFN_GATE_INP: if (d.experts > 0) r = hy_put_rows(ctx, L.router, 0, d.experts, W, host, bytes, type, 0); break;
-        case GL3_T_FFN_GATE_INP_SHEXP: if (d.experts > 0 && d.shared_ff > 0) r = hy_put_rows(ctx, L.router, d.experts, 1, W, host, bytes, type, 0); break;
+        case GL3_T_FFN_GATE_INP_SHEXP: if (d.experts > 0 && d.shared_ff > 0 && !d.shared_ungated) r = hy_put_rows(ctx, L.router, d.experts, 1, W, host, bytes, type, 0); break;
         case GL3_T_FFN_GATE_EXPS: case GL3_T_FFN_UP_EXPS:
             if (d.experts > 0) {
                 const size_t per = (size_t)d.ff * W * tes;
@@ -580,7 +666,11 @@ static uint64_t hy_needed(const gl3_hybrid_state* h, const gl3_layer_desc& d, bo
     if (!h->plain) m |= (1ull << GL3_T_HC1_IN) | (1ull << GL3_T_HC1_OUT) | (1ull << GL3_T_HC1_MIX);
     if (h->depth) m |= 1ull << GL3_T_DEPTH_MIX;
     if (h->side_dim > 0) m |= (1ull << GL3_T_SIDE_GATE) | (1ull << GL3_T_SIDE_PROJ) | (1ull << GL3_T_SIDE_NORM);
-    if (d.mixer == GL3_MIX_LATENT) m |= (1ull << GL3_T_WQ) | (1ull << GL3_T_KV_DOWN) | (1ull << GL3_T_KV_DOWN_NORM) | (1ull << GL3_T_K_UP) | (1ull << GL3_T_V_UP);
+    if (d.mixer == GL3_MIX_LATENT) m |= (1ull << GL3_T_WQ) | (1ull << GL3_T_K_UP) | (1ull << GL3_T_V_UP);
+    if (d.mixer == GL3_MIX_LATENT && d.kv_share == 0) m |= (1ull << GL3_T_KV_DOWN) | (1ull << GL3_T_KV_DOWN_NORM);
+    if (d.mixer == GL3_MIX_LATENT && d.q_rank > 0) m |= (1ull << GL3_T_Q_DOWN) | (1ull << GL3_T_Q_DOWN_NORM);
+    if (h->post_norms) m |= (1ull << GL3_T_ATTN_POST_NORM) | (d.ff > 0 ? 1ull << GL3_T_FFN_POST_NORM : 0);
+    if (d.experts > 0 && d.route_bias) m |= 1ull << GL3_T_FFN_ROUTE_BIAS;
     if ((d.mixer == GL3_MIX_ATTENTION || d.mixer == GL3_MIX_LATENT) && d.out_gate) m |= 1ull << GL3_T_ATTN_GATE;
     if (d.mixer == GL3_MIX_SSM)
         m |= (1ull << GL3_T_SSM_IN) | (1ull << GL3_T_SSM_CONV) | (1ull << GL3_T_SSM_CONV_BIAS) | (1ull << GL3_T_SSM_DT_BIAS) | (1ull << GL3_T_SSM_A_LOG) |
@@ -588,8 +678,8 @@ static uint64_t hy_needed(const gl3_hybrid_state* h, const gl3_layer_desc& d, bo
     if (d.ff > 0 && !h->parallel) m |= 1ull << GL3_T_FFN_NORM;
     if (d.ff > 0 && !h->plain) m |= (1ull << GL3_T_HC2_IN) | (1ull << GL3_T_HC2_OUT) | (1ull << GL3_T_HC2_MIX);
     if (d.experts > 0) m |= (1ull << GL3_T_FFN_GATE_INP) | (1ull << GL3_T_FFN_GATE_EXPS) | (1ull << GL3_T_FFN_UP_EXPS) | (1ull << GL3_T_FFN_DOWN_EXPS);
-    if (d.experts > 0 && d.shared_ff > 0) m |= 1ull << GL3_T_FFN_GATE_INP_SHEXP;
-    if (d.experts > 0 ? d.shared_ff > 0 : d.ff > 0) m |= (1ull << GL3_T_W1) | (1ull << GL3_T_W2) | (1ull << GL3_T_W3);
+    if (d.experts > 0 && d.shared_ff > 0 && !d.shared_ungated) m |= 1ull << GL3_T_FFN_GATE_INP_SHEXP;
+    if (d.experts > 0 ? d.shared_ff > 0 : d.ff > 0) m |= (1ull << GL3_T_W2) | (1ull << GL3_T_W3) | ((d.experts > 0 || d.ff_act != 2) ? 1ull << GL3_T_W1 : 0);
     return m;
 }
 
@@ -636,7 +726,7 @@ static void hy_gemm(gl3_ctx* ctx, const T* A, int lda, const HyMat& w, int M, fl
 #define HY_MV2(MT, KS)                                                                                                                              \
     do {                                                                                                                                            \
         if (glu) hipLaunchKernelGGL((hy_matvec_kernel<T, T, MT, HY_EPI_GLU, KS>), dim3(wgs), dim3(256), 0, st, A, lda, Wt, w.ld, M, N, K, C, ldc, act, ld_act, gp);   \
-        else if (gp.mul_table) hipLaunchKernelGGL((hy_matvec_kernel<T, T, MT, HY_EPI_ACTMUL, KS>), dim3(wgs), dim3(256), 0, st, A, lda, Wt, w.ld, M, N, K, C, ldc, act, ld_act, gp);   \
+        else if (gp.mul_table || gp.act == 2) hipLaunchKernelGGL((hy_matvec_kernel<T, T, MT, HY_EPI_ACTMUL, KS>), dim3(wgs), dim3(256), 0, st, A, lda, Wt, w.ld, M, N, K, C, ldc, act, ld_act, gp);   \
         else hipLaunchKernelGGL((hy_matvec_kernel<T, T, MT, HY_EPI_STORE, KS>), dim3(wgs), dim3(256), 0, st, A, lda, Wt, w.ld, M, N, K, C, ldc, act, ld_act, gp);    \
     } while (0)
 #define HY_MV(MT) do { if (ksplit) HY_MV2(MT, 4); else HY_MV2(MT, 1); } while (0)
@@ -649,7 +739,7 @@ static void hy_gemm(gl3_ctx* ctx, const T* A, int lda, const HyMat& w, int M, fl
     const bool big = tiles >= 256 || (parts && tiles >= 64);
     constexpr int BKT = HyPiece<T>::N * HyPiece<T>::PPR;
     int ks = 1;                                              // few result tiles and a long K: split K over blockIdx.z, the caller adds the parts
-    if (parts && !glu && !gp.mul_table && tiles < 192 && K >= 16 * BKT) ks = (int)std::min<long>(max_parts, std::max<long>(1, 256 / tiles));
+    if (parts && !glu && !gp.mul_table && gp.act != 2 && tiles < 192 && K >= 16 * BKT) ks = (int)std::min<long>(max_parts, std::max<long>(1, 256 / tiles));
     const int kper = hy_cdiv(hy_cdiv(K, ks), BKT) * BKT;
     ks = hy_cdiv(K, kper);
     if (parts) *parts = ks;
@@ -657,7 +747,7 @@ static void hy_gemm(gl3_ctx* ctx, const T* A, int lda, const HyMat& w, int M, fl
     do {                                                                                                                                            \
         const dim3 grid(hy_cdiv(N, 128), hy_cdiv(M, BM), ks);                                                                                         \
         if (glu) hipLaunchKernelGGL((hy_gemm_kernel<T, T, BM, 128, HY_EPI_GLU>), grid, dim3(256), 0, st, A, lda, Wt, w.ld, M, N, K, C, ldc, act, ld_act, gp, kper);    \
-        else if (gp.mul_table) hipLaunchKernelGGL((hy_gemm_kernel<T, T, BM, 128, HY_EPI_ACTMUL>), grid, dim3(256), 0, st, A, lda, Wt, w.ld, M, N, K, C, ldc, act, ld_act, gp, kper);    \
+        else if (gp.mul_table || gp.act == 2) hipLaunchKernelGGL((hy_gemm_kernel<T, T, BM, 128, HY_EPI_ACTMUL>), grid, dim3(256), 0, st, A, lda, Wt, w.ld, M, N, K, C, ldc, act, ld_act, gp, kper);    \
         else hipLaunchKernelGGL((hy_gemm_kernel<T, T, BM, 128, HY_EPI_STORE>), grid, dim3(256), 0, st, A, lda, Wt, w.ld, M, N, K, C, ldc, act, ld_act, gp, kper);     \
     } while (0)
     if (big) HY_GM(128); else HY_GM(64);
@@ -797,21 +887,41 @@ static int32_t hy_mixer_core(gl3_ctx* ctx, HyLayer& L, int np, int ldo, int n, i
         a.qsrc = h->proj; a.ldq = np; a.q_off = L.q_off; a.q_hstride = d.dim;
         a.xsrc = h->proj; a.ldx = np; a.x_off = L.v_off;
         a.k_mul = d.mem_k_mul != 0.f ? d.mem_k_mul : 1.f; a.q_mul = d.mem_q_mul != 0.f ? d.mem_q_mul : 1.f;
+        a.act = d.mem_qkv_act;
         a.rot = HyScanRot{d.rot_dims, L.rot_freq, d.rot_interleaved};
         a.mode = eg ? 1 : 2; a.ga = ga; a.gb = gb; a.decay = L.decay; a.ones_col = eg ? 1 : 0;
         a.heads = d.heads; a.P = P; a.N = d.dim; a.G = d.heads;
         a.state = h->slots + L.off_state; a.slot_stride = h->slot_floats; a.dyn = h->dyn; a.n = n; a.y = h->ssm_y; a.ldy = ldy;
         hy_scan(ctx, a);
-        if (n <= 32 && d.vdim > 128)
+        if (d.mem_norm_whole && !eg) {          // one norm over the heads side by side: the kernel's "head" is the token's whole row
+            if (n <= 32 && ldy > 128)
+                hipLaunchKernelGGL((hy_mem_out_kernel<T, 256>), dim3(n, 1), dim3(256), 0, st, h->ssm_y, ldy, ldy, ldy, (const float*)nullptr, 1,
+                                   d.mem_norm_weight ? L.ssm_norm : nullptr, h->proj, np, L.g_off, d.mem_gate_act, eps, L.out_mul, mixo, ldo);
+            else
+                hipLaunchKernelGGL((hy_mem_out_kernel<T, 64>), dim3(n, 1), dim3(64), 0, st, h->ssm_y, ldy, ldy, ldy, (const float*)nullptr, 1,
+                                   d.mem_norm_weight ? L.ssm_norm : nullptr, h->proj, np, L.g_off, d.mem_gate_act, eps, L.out_mul, mixo, ldo);
+        } else if (n <= 32 && d.vdim > 128)
             hipLaunchKernelGGL((hy_mem_out_kernel<T, 256>), dim3(n, d.heads), dim3(256), 0, st, h->ssm_y, ldy, P, d.vdim, eg ? ge : nullptr, d.heads,
                                d.mem_norm_weight ? L.ssm_norm : nullptr, h->proj, np, L.g_off, d.mem_gate_act, eps, L.out_mul, mixo, ldo);
         else
             hipLaunchKernelGGL((hy_mem_out_kernel<T, 64>), dim3(n, d.heads), dim3(64), 0, st, h->ssm_y, ldy, P, d.vdim, eg ? ge : nullptr, d.heads,
                                d.mem_norm_weight ? L.ssm_norm : nullptr, h->proj, np, L.g_off, d.mem_gate_act, eps, L.out_mul, mixo, ldo);
     } else if (d.mixer == GL3_MIX_LATENT) {
+        // De entries per query / key head, Re per cached row (= dim, kv_rank without a rotated part)
         float* cc = h->slots + L.off_k;
-        const int R = d.kv_rank;
-        hipLaunchKernelGGL(hy_latent_norm_kernel, dim3(n), dim3(64), 0, st, h->proj, np, L.c_off, R, L.lat_norm, eps, cc, h->slot_floats, h->dyn);
+        const int R = L.Re, De = L.De;
+        float* q = h->proj + L.q_off;
+        int ldq = np;
+        if (d.q_rank > 0) {          // queries through their own latent: norm with weight, then the expansion
+            hipLaunchKernelGGL((hy_rownorm_kernel<T>), dim3(n), dim3(256), 0, st, h->proj, np, L.q_off, d.q_rank, L.qlat_norm, eps, (T*)h->cq, d.q_rank);
+            q = h->qfull; ldq = d.heads * De;
+            hy_gemm<T>(ctx, (const T*)h->cq, d.q_rank, L.uq, n, q, ldq, false, nullptr, 0, HyGlu{});
+        }
+        if (d.rot_dim > 0)
+            hipLaunchKernelGGL(hy_latent_prep_kernel, dim3(n, 1 + d.heads), dim3(64), 0, st, q, ldq, d.dim, d.rot_dim, h->proj, np, L.c_off, d.kv_rank, L.lat_norm, eps,
+                               d.kv_share > 0 ? (float*)nullptr : cc, h->slot_floats, h->dyn, L.rot_freq, L.rot_mscale);
+        else if (d.kv_share == 0)
+            hipLaunchKernelGGL(hy_latent_norm_kernel, dim3(n), dim3(64), 0, st, h->proj, np, L.c_off, R, L.lat_norm, eps, cc, h->slot_floats, h->dyn);
         if (n > 8) {
             // A portion of many tokens: keys and values of every position so far are expanded from the slot's latents by two float32 GEMMs
             // into plan scratch (nothing but the latent is kept), and the attention core runs over them with one key / value head per
@@ -819,22 +929,22 @@ static int32_t hy_mixer_core(gl3_ctx* ctx, HyLayer& L, int np, int ldo, int n, i
             const int M = pos0 + n;
             const float* lat = cc + (size_t)seq * h->slot_floats;
             HyMat wkm, wvm;
-            wkm.w = L.wk; wkm.rows = d.heads * d.dim; wkm.k = R; wkm.ld = R;
+            wkm.w = L.wk; wkm.rows = d.heads * De; wkm.k = R; wkm.ld = R;
             wvm.w = L.wv; wvm.rows = d.heads * d.vdim; wvm.k = R; wvm.ld = R;
-            hy_gemm<float>(ctx, lat, R, wkm, M, h->kx, d.heads * d.dim, false, nullptr, 0, HyGlu{});
+            hy_gemm<float>(ctx, lat, R, wkm, M, h->kx, d.heads * De, false, nullptr, 0, HyGlu{});
             hy_gemm<float>(ctx, lat, R, wvm, M, h->vx, d.heads * d.vdim, false, nullptr, 0, HyGlu{});
-            int32_t r = hy_attention(ctx, h->proj + L.q_off, np, h->kx, h->vx, d.heads, d.heads, d.dim, d.vdim, d.scale, 0.f, n, pos0, &nsplit, false);
+            int32_t r = hy_attention(ctx, q, ldq, h->kx, h->vx, d.heads, d.heads, De, d.vdim, d.scale, 0.f, n, pos0, &nsplit, false);
             if (r != GL3_OK) return r;
             hipLaunchKernelGGL((hy_attn_merge_kernel<T>), dim3(n, d.heads), dim3(64), 0, st, h->part_acc, h->part_ml, d.heads, d.vdim, nsplit, d.softmax_sink,
-                               d.out_gate ? h->proj + L.g_off : nullptr, np, 1, mixo, ldo, (const float*)nullptr, h->dyn);
+                               d.out_gate ? h->proj + L.g_off : nullptr, np, d.out_gate == 2 ? 2 : 1, mixo, ldo, (const float*)nullptr, h->dyn);
         } else {
             // A few tokens (decode): the query is carried into the latent's space and the attention core reads the latents themselves
             // (one shared key / value head, keys = values), then the weighted sum of latents is expanded.
             if (n == 1)
-                hipLaunchKernelGGL((hy_headmm_kernel<float, 1>), dim3(1, d.heads, hy_cdiv(R, 64)), dim3(256), 0, st, h->proj + L.q_off, np, d.dim, R, L.wk,
+                hipLaunchKernelGGL((hy_headmm_kernel<float, 1>), dim3(1, d.heads, hy_cdiv(R, 64)), dim3(256), 0, st, q, ldq, De, R, L.wk,
                                    (const float*)nullptr, 0, h->qa, d.heads * R, n);
             else
-                hipLaunchKernelGGL((hy_headmm_kernel<float, 8>), dim3(hy_cdiv(n, 8), d.heads, hy_cdiv(R, 64)), dim3(256), 0, st, h->proj + L.q_off, np, d.dim, R, L.wk,
+                hipLaunchKernelGGL((hy_headmm_kernel<float, 8>), dim3(hy_cdiv(n, 8), d.heads, hy_cdiv(R, 64)), dim3(256), 0, st, q, ldq, De, R, L.wk,
                                    (const float*)nullptr, 0, h->qa, d.heads * R, n);
             int32_t r = hy_attention(ctx, h->qa, d.heads * R, cc, cc, d.heads, 1, R, R, d.scale, 0.f, n, pos0, &nsplit);
             if (r != GL3_OK) return r;
@@ -842,10 +952,10 @@ static int32_t hy_mixer_core(gl3_ctx* ctx, HyLayer& L, int np, int ldo, int n, i
                                (const float*)nullptr, 0, 0, h->oc, d.heads * R, (const float*)nullptr, h->dyn);
             if (n == 1)
                 hipLaunchKernelGGL((hy_headmm_kernel<T, 1>), dim3(1, d.heads, hy_cdiv(d.vdim, 64)), dim3(256), 0, st, h->oc, d.heads * R, R, d.vdim, L.wvT,
-                                   d.out_gate ? h->proj + L.g_off : nullptr, np, mixo, ldo, n);
+                                   d.out_gate ? h->proj + L.g_off : nullptr, np, mixo, ldo, n, d.out_gate == 2 ? 2 : 1);
             else
                 hipLaunchKernelGGL((hy_headmm_kernel<T, 8>), dim3(hy_cdiv(n, 8), d.heads, hy_cdiv(d.vdim, 64)), dim3(256), 0, st, h->oc, d.heads * R, R, d.vdim, L.wvT,
-                                   d.out_gate ? h->proj + L.g_off : nullptr, np, mixo, ldo, n);
+                                   d.out_gate ? h->proj + L.g_off : nullptr, np, mixo, ldo, n, d.out_gate == 2 ? 2 : 1);
         }
     } else {
         const int inner = d.heads * d.vdim, ch = hy_conv_ch(d), dt_off = 2 * inner + 2 * d.groups * d.state;
@@ -926,25 +1036,40 @@ static void hy_moe(gl3_ctx* ctx, HyLayer& L, int n) {
     hy_gemm<T>(ctx, hb, W, L.router, n, h->moe_z, RZ, false, nullptr, 0, HyGlu{}, &zparts, HY_ZSPLIT);
     const bool few = n <= 8;
     const int max_tiles = P / HY_MOE_BM + std::min(E, P);
+    const bool on_out = d.route_on_output != 0;          // the weights multiply the experts' outputs (in the residual update) instead of their inputs
     hipLaunchKernelGGL(hy_route_kernel, dim3(n), dim3(64), 0, st, h->moe_z, RZ, zparts, (size_t)n * RZ, E, top, h->sel, h->wsel, few ? h->pair_row : nullptr,
-                       d.shared_ff > 0 ? h->sgz : nullptr);
+                       (d.shared_ff > 0 && !d.shared_ungated) ? h->sgz : nullptr, HyRoute{d.route_softmax, L.route_bias, d.route_renorm, d.route_scale != 0.f ? d.route_scale : 1.f});
     HyMat one_gu = L.egu, one_down = L.edown;
     one_gu.rows = 2 * L.eff_pad; one_down.rows = W;
     if (few) {
         // a few tokens: the pairs of a token read its normed row themselves and the score multiplies the products (W (s h) = s (W h))
         hy_gemm_grouped<T>(ctx, hb, W, one_gu, (size_t)2 * L.eff_pad * L.egu.ld, P, max_tiles, true, nullptr, 0, true, (T*)h->eact, L.eff_pad,
-                           HyGlu{d.ff_limit, d.ff_alpha, d.ff_shift}, top, h->wsel);
+                           HyGlu{d.ff_limit, d.ff_alpha, d.ff_shift, nullptr, nullptr, 0, 0, d.ff_act}, top, on_out ? nullptr : h->wsel);
     } else {
         hipLaunchKernelGGL(hy_moe_group_kernel, dim3(1), dim3(256), (size_t)2 * E * 4, st, h->sel, P, E, HY_MOE_BM, h->pair_row, h->tiles, h->ntiles);
-        hipLaunchKernelGGL((hy_moe_scale_kernel<T>), dim3(P), dim3(256), 0, st, hb, W, top, h->wsel, h->pair_row, (T*)h->ea);
+        hipLaunchKernelGGL((hy_moe_scale_kernel<T>), dim3(P), dim3(256), 0, st, hb, W, top, on_out ? (const float*)nullptr : h->wsel, h->pair_row, (T*)h->ea);
         hy_gemm_grouped<T>(ctx, (const T*)h->ea, W, one_gu, (size_t)2 * L.eff_pad * L.egu.ld, P, max_tiles, false, nullptr, 0, true, (T*)h->eact, L.eff_pad,
-                           HyGlu{d.ff_limit, d.ff_alpha, d.ff_shift});
+                           HyGlu{d.ff_limit, d.ff_alpha, d.ff_shift, nullptr, nullptr, 0, 0, d.ff_act});
     }
     hy_gemm_grouped<T>(ctx, (const T*)h->eact, L.eff_pad, one_down, (size_t)W * L.edown.ld, P, max_tiles, few, h->eout, W, false, nullptr, 0, HyGlu{});
     if (d.shared_ff > 0) {
         T* act = (T*)h->mixo;
         hy_gemm<T>(ctx, hb, W, L.gu, n, nullptr, 0, true, act, L.ff_pad, hy_ff_glu(L));
         hy_gemm<T>(ctx, act, L.ff_pad, L.down, n, h->y, W, false, nullptr, 0, HyGlu{}, &h->y_parts);
+    }
+}
+
+// logits of the nw rows listed in h->want: final norm of the gathered rows, the head's product, the optional cap * tanh(. / cap)
+template <typename T>
+static void hy_logits(gl3_ctx* ctx, int nw) {
+    gl3_hybrid_state* h = ctx->hy;
+    T* xw = (T*)h->xw;
+    hy_streams<T>(ctx, nw, h->X, h->W, h->S, (size_t)h->mb * h->W, (const float*)nullptr, 1, 0, (const float*)nullptr, (const float*)nullptr,
+                  h->ones, h->final_norm, ctx->d.rms_eps, xw, (float*)nullptr, h->want);
+    hy_gemm<T>(ctx, xw, h->W, h->head, nw, h->logits, ctx->d.vocab, false, nullptr, 0, HyGlu{});
+    if (h->softcap > 0.f) {
+        const size_t cnt = (size_t)nw * ctx->d.vocab;
+        hipLaunchKernelGGL(hy_softcap_kernel, dim3((unsigned)std::min<size_t>(1024, (cnt + 255) / 256)), dim3(256), 0, ctx->stream, h->logits, cnt, h->softcap);
     }
 }
 
@@ -1027,29 +1152,31 @@ static int32_t hy_portion_plain(gl3_ctx* ctx, int seq, const int32_t* tokens, in
             hy_resid<T>(ctx, n, r, (T*)nullptr, hb);
             continue;
         }
+        r.post_w = L.norm1b;          // null without post norms
         if (L.d.ff > 0) {
             r.norm_w = L.norm2;
             hy_resid<T>(ctx, n, r, (T*)nullptr, hb);
             r = base;
+            r.post_w = L.norm2b;
             if (L.d.experts > 0) {
                 hy_moe<T>(ctx, L, n);
                 r.eo = h->eout; r.pair_row = h->pair_row; r.top = L.d.top;
-                if (L.d.shared_ff > 0) { r.ya = h->y; r.ya_parts = h->y_parts; r.ya_stride = (size_t)n * W; r.gate_z = h->sgz; r.gate_ld = 1; }
+                if (L.d.route_on_output) r.ew = h->wsel;
+                if (L.d.shared_ff > 0) {
+                    r.ya = h->y; r.ya_parts = h->y_parts; r.ya_stride = (size_t)n * W;
+                    if (!L.d.shared_ungated) { r.gate_z = h->sgz; r.gate_ld = 1; }
+                }
             } else {
                 T* act = (T*)h->mixo;
-                hy_gemm<T>(ctx, hb, W, L.gu, n, nullptr, 0, true, act, L.ff_pad, hy_ff_glu(L));
+                if (L.d.ff_act == 2) hy_gemm<T>(ctx, hb, W, L.gu, n, nullptr, 0, false, act, L.ff_pad, HyGlu{0.f, 0.f, 0.f, nullptr, nullptr, 0, 0, 2});      // no gate: relu(up)^2
+                else hy_gemm<T>(ctx, hb, W, L.gu, n, nullptr, 0, true, act, L.ff_pad, hy_ff_glu(L));
                 hy_gemm<T>(ctx, act, L.ff_pad, L.down, n, h->y, W, false, nullptr, 0, HyGlu{}, &h->y_parts);
                 r.ya = h->y; r.ya_parts = h->y_parts; r.ya_stride = (size_t)n * W;
             }
         }
         finish(r);
     }
-    if (nw > 0) {
-        T* xw = (T*)h->xw;
-        hy_streams<T>(ctx, nw, h->X, W, 1, lstride, (const float*)nullptr, 1, 0, (const float*)nullptr, (const float*)nullptr,
-                           h->ones, h->final_norm, eps, xw, (float*)nullptr, h->want);
-        hy_gemm<T>(ctx, xw, W, h->head, nw, h->logits, ctx->d.vocab, false, nullptr, 0, HyGlu{});
-    }
+    if (nw > 0) hy_logits<T>(ctx, nw);
     HY_HIP(hipGetLastError());
     return GL3_OK;
 }
@@ -1092,12 +1219,7 @@ static int32_t hy_portion(gl3_ctx* ctx, int seq, const int32_t* tokens, int n, i
                                h->taps ? h->taps + (size_t)l * sstride : nullptr, (const int*)nullptr);
         }
     }
-    if (nw > 0) {
-        T* xw = (T*)h->xw;
-        hy_streams<T>(ctx, nw, h->X, W, S, sstride, (const float*)nullptr, 1, 0, (const float*)nullptr, (const float*)nullptr,
-                           h->ones, h->final_norm, eps, xw, (float*)nullptr, h->want);
-        hy_gemm<T>(ctx, xw, W, h->head, nw, h->logits, ctx->d.vocab, false, nullptr, 0, HyGlu{});
-    }
+    if (nw > 0) hy_logits<T>(ctx, nw);
     HY_HIP(hipGetLastError());
     return GL3_OK;
 }
@@ -1138,18 +1260,9 @@ int32_t gl3_hy_step(gl3_ctx* ctx, int32_t seq, const int32_t* tokens, int32_t n,
                                : hy_portion<bf16_t>(ctx, seq, tokens + off, pn, start_pos + off, rel.data(), g);
                 ran = true;
             } else {
-                const int W = h->W, S = h->S;
                 memcpy(h->h_want, rel.data(), (size_t)g * 4);
                 HY_HIP(hipMemcpyAsync(h->want, h->h_want, (size_t)g * 4, hipMemcpyHostToDevice, ctx->stream));
-                if (h->f32) {
-                    hy_streams<float>(ctx, g, h->X, W, S, (size_t)h->mb * W, (const float*)nullptr, 1, 0, (const float*)nullptr,
-                                       (const float*)nullptr, h->ones, h->final_norm, ctx->d.rms_eps, (float*)h->xw, (float*)nullptr, h->want);
-                    hy_gemm<float>(ctx, (float*)h->xw, W, h->head, g, h->logits, ctx->d.vocab, false, nullptr, 0, HyGlu{});
-                } else {
-                    hy_streams<bf16_t>(ctx, g, h->X, W, S, (size_t)h->mb * W, (const float*)nullptr, 1, 0, (const float*)nullptr,
-                                       (const float*)nullptr, h->ones, h->final_norm, ctx->d.rms_eps, (bf16_t*)h->xw, (float*)nullptr, h->want);
-                    hy_gemm<bf16_t>(ctx, (bf16_t*)h->xw, W, h->head, g, h->logits, ctx->d.vocab, false, nullptr, 0, HyGlu{});
-                }
+                if (h->f32) hy_logits<float>(ctx, g); else hy_logits<bf16_t>(ctx, g);
                 r = GL3_OK;
             }
             if (r != GL3_OK) return r;

@@ -460,7 +460,133 @@ bool kosusun_tensor(const std::string& name, int32_t& id, int32_t& layer, int32_
     return true;
 }
 
-const Design DESIGNS[] = {{"Noditar", noditar_describe, noditar_tensor}, {"Vonulix", vonulix_describe, vonulix_tensor}, {"Kosusun", kosusun_describe, kosusun_tensor}};
+// Kugadra: one plain residual stream with a norm in front of AND behind every sublayer, x <- x + rms_norm(sublayer(rms_norm(x, w)), w_post).
+// Two layer types.  "lightning": a matrix memory with a fixed decay per head behind silu-activated q / k / v (no rotation, no other
+// scale), the heads side by side through ONE RMS norm with a weight, times sigmoid(W_g h).  "latent_attention": queries through a normed
+// latent of their own, keys and values expanded from a cached normed latent, a rotated part of rot_dim entries per query head and one
+// rotated key part for all heads (half-split pairs, frequencies blended towards / factor along a ramp over the pair index, cos and sin
+// times 0.1 ln(factor) + 1), causal softmax, one sigmoid gate per head; a layer with "kv_from" reads that layer's cache.  Feed-forward:
+// dense = W_down relu(W_up h)^2, or a mixture of silu-gated experts (softmax scores over all experts, chosen by score + a correction,
+// weights = the chosen scores renormalised (+ 1e-20) times router.scale, applied to the experts' outputs) plus an ungated shared
+// expert.  The head is the embedding table; logits pass cap * tanh(. / cap).  config.json gives every size and the constants named
+// here; the forms are the design's and are fixed here.
+bool kugadra_describe(const JVal& cfg, gl3_model_desc& d, std::vector<gl3_layer_desc>& layers, DescStore& store, std::string& err) {
+    d.arch = GL3_ARCH_LAYERLIST;
+    d.weight_type = GL3_TYPE_BF16;
+    if (!get_int(cfg, "vocab", d.vocab, err) || !get_int(cfg, "width", d.dim, err)) return false;
+    d.streams = 0;
+    d.post_norms = 1;
+    d.embedding_scale = 1.f;
+    if (const JVal* e = cfg.get("embedding"))
+        if (e->kind == JVal::OBJ && e->get("scale") && !get_float(*e, "scale", d.embedding_scale, err)) return false;
+    if (const JVal* cap = cfg.get("logit_softcap"))
+        if (!cap->is_null() && !get_float(cfg, "logit_softcap", d.logit_softcap, err)) return false;
+    const JVal* norm = cfg.get("norm");
+    if (!norm || !get_float(*norm, "eps", d.rms_eps, err)) { if (err.empty()) err = "config: missing norm.eps"; return false; }
+    const JVal* ls = cfg.get("layers");
+    if (!ls || ls->kind != JVal::ARR || ls->arr.empty()) { err = "config: 'layers' must be a non-empty list"; return false; }
+    for (const JVal& l : ls->arr) {
+        gl3_layer_desc ld{};
+        const JVal *ty = l.get("type"), *mx = l.get("mixer"), *mlp = l.get("mlp");
+        if (!ty || ty->kind != JVal::STR || !mx || mx->kind != JVal::OBJ) { err = "config: a layer needs 'type' and 'mixer'"; return false; }
+        if (!get_int(*mx, "heads", ld.heads, err) || !get_int(*mx, "dim", ld.dim, err) || !get_int(*mx, "vdim", ld.vdim, err)) return false;
+        ld.kv_heads = ld.heads;
+        if (ty->str == "lightning") {
+            ld.mixer = GL3_MIX_MEMORY;
+            ld.mem_gates = GL3_MEM_DECAY;
+            const JVal* dec = mx->get("decay");
+            if (!dec || dec->kind != JVal::ARR || (int)dec->arr.size() != ld.heads) { err = "config: lightning needs a decay per head"; return false; }
+            store.floats.emplace_back();
+            for (const JVal& v : dec->arr) {
+                if (v.kind != JVal::NUM) { err = "config: decay must be numbers"; return false; }
+                store.floats.back().push_back((float)v.num);
+            }
+            ld.mem_decay = store.floats.back().data();
+            ld.mem_qkv_act = 1; ld.mem_norm_whole = 1; ld.mem_norm_weight = 1; ld.mem_gate_act = 1;
+        } else if (ty->str == "latent_attention") {
+            ld.mixer = GL3_MIX_LATENT;
+            ld.out_gate = 2;
+            if (!get_int(*mx, "kv_rank", ld.kv_rank, err) || !get_int(*mx, "q_rank", ld.q_rank, err) || !get_int(*mx, "rot_dim", ld.rot_dim, err) ||
+                !get_float(*mx, "scale", ld.scale, err))
+                return false;
+            if (ld.q_rank < 1) { err = "config: q_rank must be positive"; return false; }
+            if (const JVal* kf = mx->get("kv_from"))
+                if (!kf->is_null()) {
+                    int32_t j = -1;
+                    if (!get_int(*mx, "kv_from", j, err)) return false;
+                    if (j < 0 || j >= (int32_t)layers.size()) { err = "config: kv_from must name an earlier layer"; return false; }
+                    ld.kv_share = j + 1;
+                }
+            if (ld.rot_dim > 0) {
+                const JVal* rot = mx->get("rot");
+                int32_t dims = 0;
+                if (!rot || rot->kind != JVal::OBJ || !get_int(*rot, "dims", dims, err) || !get_float(*rot, "base", ld.rot_base, err)) {
+                    if (err.empty()) err = "config: a latent attention with rot_dim needs rot.dims and rot.base";
+                    return false;
+                }
+                if (dims != ld.rot_dim) { err = "config: rot.dims must equal rot_dim"; return false; }
+                if (const JVal* sc = rot->get("scaling"))
+                    if (sc->kind == JVal::OBJ &&
+                        (!get_float(*sc, "factor", ld.rot_yarn_factor, err) || !get_float(*sc, "original", ld.rot_yarn_original, err) ||
+                         !get_float(*sc, "fast", ld.rot_yarn_fast, err) || !get_float(*sc, "slow", ld.rot_yarn_slow, err)))
+                        return false;
+            }
+        } else { err = "config: unknown layer type '" + ty->str + "'"; return false; }
+        if (mlp && !mlp->is_null()) {
+            const JVal* kind = mlp->get("kind");
+            if (!kind || kind->kind != JVal::STR) { err = "config: mlp needs 'kind'"; return false; }
+            if (kind->str == "dense") {
+                if (!get_int(*mlp, "ff", ld.ff, err)) return false;
+                ld.ff_act = 2;
+            } else if (kind->str == "moe") {
+                const JVal *ex = mlp->get("expert"), *ro = mlp->get("router"), *sh = mlp->get("shared");
+                if (!ex || !ro || !get_int(*ex, "ff", ld.ff, err) || !get_int(*ro, "experts", ld.experts, err) || !get_int(*ro, "top", ld.top, err)) {
+                    if (err.empty()) err = "config: a mixture of experts needs 'expert' and 'router'";
+                    return false;
+                }
+                ld.route_scale = 1.f;
+                if (ro->get("scale") && !get_float(*ro, "scale", ld.route_scale, err)) return false;
+                if (sh && !sh->is_null() && !get_int(*sh, "ff", ld.shared_ff, err)) return false;
+                ld.ff_alpha = 1.f; ld.ff_shift = 0.f;          // silu(g) u
+                ld.route_softmax = 1; ld.route_bias = 1; ld.route_renorm = 1; ld.route_on_output = 1; ld.shared_ungated = 1;
+            } else { err = "config: mlp.kind must be 'dense' or 'moe'"; return false; }
+        }
+        layers.push_back(ld);
+    }
+    d.n_layers = (int32_t)layers.size();
+    return true;
+}
+
+bool kugadra_tensor(const std::string& name, int32_t& id, int32_t& layer, int32_t& expert) {
+    static const std::map<std::string, int> global = {{"embed", GL3_T_TOKEN_EMBD}, {"final.norm", GL3_T_OUTPUT_NORM}};
+    static const std::map<std::string, int> leaf = {
+        {"norm1", GL3_T_ATTN_NORM}, {"norm2", GL3_T_FFN_NORM}, {"norm1b", GL3_T_ATTN_POST_NORM}, {"norm2b", GL3_T_FFN_POST_NORM},
+        {"mix.q", GL3_T_WQ}, {"mix.k", GL3_T_WK}, {"mix.v", GL3_T_WV}, {"mix.g", GL3_T_ATTN_GATE}, {"mix.o", GL3_T_WO}, {"mix.norm", GL3_T_SSM_NORM},
+        {"mix.dq", GL3_T_Q_DOWN}, {"mix.dq.norm", GL3_T_Q_DOWN_NORM}, {"mix.uq", GL3_T_WQ}, {"mix.dkv", GL3_T_KV_DOWN}, {"mix.dkv.norm", GL3_T_KV_DOWN_NORM},
+        {"mix.uk", GL3_T_K_UP}, {"mix.uv", GL3_T_V_UP}, {"mlp.up", GL3_T_W3}, {"mlp.down", GL3_T_W2}, {"mlp.router", GL3_T_FFN_GATE_INP},
+        {"mlp.correction", GL3_T_FFN_ROUTE_BIAS}, {"mlp.shared.gate", GL3_T_W1}, {"mlp.shared.up", GL3_T_W3}, {"mlp.shared.down", GL3_T_W2}};
+    static const std::map<std::string, int> part = {{"gate", GL3_T_FFN_GATE_EXPS}, {"up", GL3_T_FFN_UP_EXPS}, {"down", GL3_T_FFN_DOWN_EXPS}};
+    expert = -1;
+    auto g = global.find(name);
+    if (g != global.end()) { id = g->second; layer = 0; return true; }
+    std::string lf;
+    if (!split_layer_name(name, layer, lf)) return false;
+    auto f = leaf.find(lf);
+    if (f != leaf.end()) { id = f->second; return true; }
+    if (lf.compare(0, 5, "mlp.e") == 0) {          // mlp.e<k>.gate | up | down
+        size_t i = 5;
+        while (i < lf.size() && lf[i] >= '0' && lf[i] <= '9') ++i;
+        if (i == 5 || i > 12 || i >= lf.size() || lf[i] != '.') return false;
+        auto pf = part.find(lf.substr(i + 1));
+        if (pf == part.end()) return false;
+        id = pf->second; expert = atoi(lf.substr(5, i - 5).c_str());
+        return true;
+    }
+    return false;
+}
+
+const Design DESIGNS[] = {{"Noditar", noditar_describe, noditar_tensor}, {"Vonulix", vonulix_describe, vonulix_tensor}, {"Kosusun", kosusun_describe, kosusun_tensor},
+                          {"Kugadra", kugadra_describe, kugadra_tensor}};
 
 struct Mapping {
     void* p = MAP_FAILED; size_t n = 0;

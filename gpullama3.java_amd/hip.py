@@ -61,7 +61,11 @@ class LayerDesc(C.Structure):
                 ("qk_bias", C.c_int32), ("rot_interleaved", C.c_int32), ("pool", C.c_int32),
                 ("mem_gates", C.c_int32), ("mem_decay", C.POINTER(C.c_float)), ("mem_q_mul", C.c_float), ("mem_k_mul", C.c_float),
                 ("mem_gate_cap", C.c_float), ("mem_norm_weight", C.c_int32), ("mem_gate_act", C.c_int32),
-                ("beside", C.c_void_p), ("out_scale", C.c_float)]          # beside: address of another LayerDesc
+                ("beside", C.c_void_p), ("out_scale", C.c_float),          # beside: address of another LayerDesc
+                ("q_rank", C.c_int32), ("rot_dim", C.c_int32), ("kv_share", C.c_int32), ("rot_yarn_factor", C.c_float),
+                ("rot_yarn_original", C.c_float), ("rot_yarn_fast", C.c_float), ("rot_yarn_slow", C.c_float),
+                ("mem_qkv_act", C.c_int32), ("mem_norm_whole", C.c_int32), ("route_softmax", C.c_int32), ("route_bias", C.c_int32),
+                ("route_renorm", C.c_int32), ("route_on_output", C.c_int32), ("shared_ungated", C.c_int32), ("route_scale", C.c_float)]
 
 
 class ModelDesc(C.Structure):
@@ -73,7 +77,8 @@ class ModelDesc(C.Structure):
                 ("residual_scale", C.c_float), ("logit_scale", C.c_float),
                 ("n_experts", C.c_int32), ("n_experts_used", C.c_int32), ("moe_hidden", C.c_int32),
                 ("streams", C.c_int32), ("layer_descs", C.POINTER(LayerDesc)),
-                ("norm_offset", C.c_float), ("side_dim", C.c_int32), ("depth_mix", C.c_int32), ("parallel_block", C.c_int32)]
+                ("norm_offset", C.c_float), ("side_dim", C.c_int32), ("depth_mix", C.c_int32), ("parallel_block", C.c_int32),
+                ("post_norms", C.c_int32), ("logit_softcap", C.c_float)]
 
 
 class KernelTimes(C.Structure):

@@ -71,7 +71,7 @@ enum { GL3_ARCH_LLAMA = 0, GL3_ARCH_QWEN3 = 1, GL3_ARCH_QWEN2 = 2,
                               * gl3_layer_desc; several residual streams mixed by per-sublayer tables, or one plain residual with an optional
                               * weighted average over all earlier layers' results; bfloat16 or float32 matrices
                               * (GL3_TYPE_BF16, GL3_FLAG_F32_COMPUTE); model folders with config.json + model.safetensors (gl3_load_model_dir) */
-       GL3_ARCH_LAYERLIST = 6 /* the same family under its own name: the registered designs (Noditar, Vonulix, Kosusun) differ only in
+       GL3_ARCH_LAYERLIST = 6 /* the same family under its own name: the registered designs (Noditar, Vonulix, Kosusun, Kugadra) differ only in
                               * the parameters of gl3_model_desc / gl3_layer_desc that their `describe` fills in */ };
 
 /* token mixers of a layer-list model (gl3_layer_desc.mixer) */
@@ -150,6 +150,29 @@ typedef struct gl3_layer_desc {
      * projection.  Its tensors are uploaded with layer + GL3_LAYER_BESIDE. */
     const struct gl3_layer_desc* beside;
     float   out_scale;
+    /* latent attention, further switches (each usable alone).
+     * q_rank > 0: queries go through a latent of their own, q = W_uq rms_norm(W_dq h) (GL3_T_Q_DOWN [q_rank x width], its norm weight
+     * GL3_T_Q_DOWN_NORM [q_rank], GL3_T_WQ = W_uq [heads (dim + rot_dim) x q_rank]); 0: q = W_q h.
+     * rot_dim > 0: every query head has rot_dim more entries behind its dim unrotated ones, GL3_T_KV_DOWN has rot_dim more rows behind its
+     * kv_rank latent rows (not normed), and these parts turn by their position (pairs i, i + rot_dim / 2; rot_base; frequencies as
+     * below); the turned key part is ONE for all heads and is cached behind the latent; score = scale (q_unrotated . W_uk c + q_rotated . k_rotated).
+     * rot_yarn_factor > 0 (also read by attention and matrix-memory mixers with rot_dims > 0): frequency f_i = rot_base^(-2 i / n) becomes
+     * f_i / factor * r_i + f_i (1 - r_i) with r_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), lo = max(floor(p(fast)), 0),
+     * hi = min(ceil(p(slow)), n - 1), p(t) = n ln(original / (2 pi t)) / (2 ln rot_base), and cos and sin are multiplied by
+     * 0.1 ln(factor) + 1.  kv_share = j + 1 > 0: the layer has no down projection and no cache rows of its own, it reads the latent
+     * rows (and turned key parts) that layer j < this layer writes (same kv_rank and rot_dim), with its own expansions. */
+    int32_t q_rank, rot_dim, kv_share;
+    float   rot_yarn_factor, rot_yarn_original, rot_yarn_fast, rot_yarn_slow;
+    /* matrix memory, further switches.  mem_qkv_act = 1: q, k and v are silu(projection).  mem_norm_whole = 1: ONE root mean square over
+     * the token's heads side by side (heads vdim entries) instead of one per head. */
+    int32_t mem_qkv_act, mem_norm_whole;
+    /* feed-forward, further switches.  ff_act = 2: no gate, act = relu(W_up h)^2 (GL3_T_W3, GL3_T_W2 only).  Mixture of experts:
+     * route_softmax = 1: scores = softmax over all experts (else sigmoid); route_bias = 1: the experts are chosen by score +
+     * GL3_T_FFN_ROUTE_BIAS [experts], the weights stay the scores; route_renorm = 1: the chosen weights are divided by their sum + 1e-20;
+     * route_scale (0 = 1) multiplies them; route_on_output = 1: a weight multiplies its expert's OUTPUT (else its input);
+     * shared_ungated = 1: the shared expert has no gate (no GL3_T_FFN_GATE_INP_SHEXP) */
+    int32_t route_softmax, route_bias, route_renorm, route_on_output, shared_ungated;
+    float   route_scale;
 } gl3_layer_desc;
 
 /* ggml tensor types of the wire format (J/tensor/GGMLType.java:5-21) */
@@ -213,7 +236,12 @@ enum {
     GL3_T_MEM_FGATE = 49,          /* matrix memory: forget gate projection          [heads x width]                     */
     GL3_T_MEM_IGATE_BIAS = 50,     /*                                                [heads]                             */
     GL3_T_MEM_FGATE_BIAS = 51,     /*                                                [heads]                             */
-    GL3_T_COUNT = 52
+    GL3_T_ATTN_POST_NORM = 52,     /* gl3_model_desc.post_norms: norm of the mixer's output          [width]             */
+    GL3_T_FFN_POST_NORM = 53,      /*                            norm of the feed-forward's output   [width]             */
+    GL3_T_Q_DOWN = 54,             /* latent: down projection of the queries         [q_rank x width]                    */
+    GL3_T_Q_DOWN_NORM = 55,        /* latent: norm weight of the query latent        [q_rank]                            */
+    GL3_T_FFN_ROUTE_BIAS = 56,     /* mixture of experts: added to the scores for the choice only    [experts]           */
+    GL3_T_COUNT = 57
 };
 
 /* gl3_model_desc.flags */
@@ -285,6 +313,11 @@ typedef struct {
      * x <- x + residual_scale (mixer(norm1 x) + ff(norm1 x)) (residual_scale, above, 0 = 1; no GL3_T_FFN_NORM).  logit_scale (above,
      * 0 = 1) multiplies the family's logits. */
     int32_t parallel_block;
+    /* layer-list family with streams == 0.  post_norms != 0: every sublayer's output is RMS-normed with a weight of its own before it
+     * joins the residual, x <- x + rms_norm(sublayer(rms_norm(x, w)), w_post) (GL3_T_ATTN_POST_NORM, GL3_T_FFN_POST_NORM).
+     * logit_softcap > 0: logits <- cap tanh(logits / cap). */
+    int32_t post_norms;
+    float   logit_softcap;
 } gl3_model_desc;
 
 /* Per-kernel-class device time of one instrumented decode step (HIP events around every launch). */
