@@ -32,6 +32,7 @@ using gl3::argmax_kernel;
 
 static inline int hy_cdiv(int a, int b) { return (a + b - 1) / b; }
 constexpr int HY_MOE_BM = 64;        // rows per tile of the grouped expert GEMMs
+constexpr int HY_LATENT_DIRECT = 512;   // longest cached latent row that decode steps score in the latent's space (value columns per lane of the attention core)
 constexpr int HY_ZSPLIT = 16;        // most K-split parts of a product with very few result rows (router, token input's gate): its consumer kernel adds them
 static inline float hy_bf16_to_f32(uint16_t v) { uint32_t u = (uint32_t)v << 16; float f; memcpy(&f, &u, 4); return f; }
 static inline uint16_t hy_f32_to_bf16(float f) {
@@ -99,7 +100,7 @@ static const char* hy_check_layer(const gl3_layer_desc& d) {
     } else if (d.mixer == GL3_MIX_LATENT) {
         if (d.dim < 1 || d.kv_rank < 1) return "latent attention: dim and kv_rank must be positive";
         if (d.rot_dim < 0 || (d.rot_dim & 1)) return "latent attention: rot_dim must be even and >= 0";
-        if (d.kv_rank + d.rot_dim > 512) return "latent attention: kv_rank + rot_dim <= 512";
+        if (d.kv_rank + d.rot_dim > 8192 || d.dim + d.rot_dim > 1024 || d.vdim > 512) return "latent attention: kv_rank + rot_dim <= 8192, dim + rot_dim <= 1024, vdim <= 512";
         if (d.rot_dim > 0 && !(d.rot_base > 0.f)) return "latent attention: rot_base must be positive";
         if (d.rot_dim > 0 && d.rot_yarn_factor > 0.f && !(d.rot_yarn_original > 0.f && d.rot_yarn_fast > 0.f && d.rot_yarn_slow > 0.f && d.rot_base != 1.f))
             return "latent attention: scaled frequencies need original, fast and slow > 0";
@@ -187,6 +188,7 @@ int32_t gl3_hy_create(const gl3_model_desc* desc, gl3_ctx** out, std::string& er
     int max_proj = 1, max_mix = W, max_ch = 1, max_inner = 1, max_hr = 1, max_hdv = 1, max_kx = 0, max_vx = 0, max_rz = 0, max_top = 0, max_eff = 0, max_e = 0;
     if (h->side_dim > 0) TRY(hy_alloc_mat(ctx, h->side_emb, V, desc->n_layers * h->side_dim, desc->n_layers * h->side_dim));
     int max_heads = 1, max_qr = 0, max_qfull = 0;
+    bool long_latent = false;
     // one mixer's share of the layer: its offsets in the fused projection row (p0 = its first row) and in mixo / o (o0 = its first
     // column), its vectors and tables, its part of the sequence slot
     auto setup_mixer = [&](HyLayer& Ly, int p0, int o0) -> int32_t {
@@ -256,7 +258,9 @@ int32_t gl3_hy_create(const gl3_model_desc* desc, gl3_ctx** out, std::string& er
                 TRYM(hy_alloc(ctx, &Ly.rot_freq, f.size() * 4));
                 if (hipMemcpy(Ly.rot_freq, f.data(), f.size() * 4, hipMemcpyHostToDevice) != hipSuccess) { ctx->err = "copy of the rotary table failed"; return GL3_E_HIP; }
             }
-            max_hr = std::max(max_hr, d.heads * Re); max_hdv = std::max(max_hdv, std::max(d.heads * Re, d.heads * d.vdim));
+            if (Re <= HY_LATENT_DIRECT) max_hr = std::max(max_hr, d.heads * Re);
+            else long_latent = true;
+            max_hdv = std::max(max_hdv, std::max(Re <= HY_LATENT_DIRECT ? d.heads * Re : 0, d.heads * d.vdim));
             max_kx = std::max(max_kx, d.heads * De); max_vx = std::max(max_vx, d.heads * d.vdim);
         } else if (d.mixer == GL3_MIX_MEMORY) {
             const bool eg = d.mem_gates == GL3_MEM_EXP_GATES;
@@ -365,7 +369,7 @@ int32_t gl3_hy_create(const gl3_model_desc* desc, gl3_ctx** out, std::string& er
         TRY(hy_alloc(ctx, &h->cq, (size_t)mb * max_qr * es));
         TRY(hy_alloc(ctx, &h->qfull, (size_t)mb * max_qfull * 4));
     }
-    if (max_kx > 0 && mb > 8) {          // latent attention, portions of many tokens: expanded keys / values of one layer at a time
+    if (max_kx > 0 && (mb > 8 || long_latent)) {          // latent attention, portions of many tokens (or cached rows too long for the latent-space form): expanded keys / values of one layer at a time
         TRY(hy_alloc(ctx, &h->kx, (size_t)C * max_kx * 4));
         TRY(hy_alloc(ctx, &h->vx, (size_t)C * max_vx * 4));
     }
@@ -922,8 +926,8 @@ static int32_t hy_mixer_core(gl3_ctx* ctx, HyLayer& L, int np, int ldo, int n, i
                                d.kv_share > 0 ? (float*)nullptr : cc, h->slot_floats, h->dyn, L.rot_freq, L.rot_mscale);
         else if (d.kv_share == 0)
             hipLaunchKernelGGL(hy_latent_norm_kernel, dim3(n), dim3(64), 0, st, h->proj, np, L.c_off, R, L.lat_norm, eps, cc, h->slot_floats, h->dyn);
-        if (n > 8) {
-            // A portion of many tokens: keys and values of every position so far are expanded from the slot's latents by two float32 GEMMs
+        if (n > 8 || R > HY_LATENT_DIRECT) {
+            // A portion of many tokens (or cached rows longer than the latent-space form below holds in registers): keys and values of every position so far are expanded from the slot's latents by two float32 GEMMs
             // into plan scratch (nothing but the latent is kept), and the attention core runs over them with one key / value head per
             // query head: 4 x less arithmetic than scoring in the latent's space when kv_rank is 4 x the head size.
             const int M = pos0 + n;

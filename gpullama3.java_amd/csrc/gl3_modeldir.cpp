@@ -506,9 +506,8 @@ bool kugadra_describe(const JVal& cfg, gl3_model_desc& d, std::vector<gl3_layer_
         } else if (ty->str == "latent_attention") {
             ld.mixer = GL3_MIX_LATENT;
             ld.out_gate = 2;
-            if (!get_int(*mx, "kv_rank", ld.kv_rank, err) || !get_int(*mx, "q_rank", ld.q_rank, err) || !get_int(*mx, "rot_dim", ld.rot_dim, err) ||
-                !get_float(*mx, "scale", ld.scale, err))
-                return false;
+            if (!get_int(*mx, "kv_rank", ld.kv_rank, err) || !get_int(*mx, "q_rank", ld.q_rank, err) || !get_float(*mx, "scale", ld.scale, err)) return false;
+            if (mx->get("rot_dim") && !mx->get("rot_dim")->is_null() && !get_int(*mx, "rot_dim", ld.rot_dim, err)) return false;
             if (ld.q_rank < 1) { err = "config: q_rank must be positive"; return false; }
             if (const JVal* kf = mx->get("kv_from"))
                 if (!kf->is_null()) {

@@ -1,4 +1,4 @@
-"""Host side of the layer-list family (GL3_ARCH_LAYERLIST: the Noditar, Vonulix and Kosusun designs) over the C-ABI: model folders (config.json + model.safetensors), the step
+"""Host side of the layer-list family (GL3_ARCH_LAYERLIST: the Noditar, Vonulix, Kosusun and Kugadra designs) over the C-ABI: model folders (config.json + model.safetensors), the step
 function with sequence slots, greedy / sampled generation.  The compute path is csrc/gl3_hybrid.hip; nothing here computes.
 
     plan = HybridPlan.from_dir("model-folder", dtype="bfloat16", ctx=4096, max_batch=512, n_seqs=2)
@@ -249,20 +249,56 @@ def kosusun_tensor_shapes(config: dict) -> dict:
     return out
 
 
+def kugadra_tensor_shapes(config: dict) -> dict:
+    """{tensor name: shape} of a Kugadra configuration, in file order (the head is the embedding table)."""
+    W, V = config["width"], config["vocab"]
+    out = {"embed": (V, W)}
+    for i, layer in enumerate(config["layers"]):
+        p, m, ff = "l%d." % i, layer["mixer"], layer.get("mlp")
+        od = m["heads"] * m["vdim"]
+        out.update({p + "norm1": (W,), p + "norm1b": (W,)})
+        if layer["type"] == "lightning":
+            out.update({p + "mix.q": (m["heads"] * m["dim"], W), p + "mix.k": (m["heads"] * m["dim"], W), p + "mix.v": (od, W), p + "mix.g": (od, W),
+                        p + "mix.o": (W, od), p + "mix.norm": (od,)})
+        else:
+            P = m.get("rot_dim", 0)
+            out.update({p + "mix.dq": (m["q_rank"], W), p + "mix.dq.norm": (m["q_rank"],), p + "mix.uq": (m["heads"] * (m["dim"] + P), m["q_rank"])})
+            if m.get("kv_from") is None:
+                out.update({p + "mix.dkv": (m["kv_rank"] + P, W), p + "mix.dkv.norm": (m["kv_rank"],)})
+            out.update({p + "mix.uk": (m["heads"] * m["dim"], m["kv_rank"]), p + "mix.uv": (od, m["kv_rank"]), p + "mix.g": (m["heads"], W), p + "mix.o": (W, od)})
+        if ff:
+            out.update({p + "norm2": (W,), p + "norm2b": (W,)})
+            if ff["kind"] == "dense":
+                out.update({p + "mlp.up": (ff["ff"], W), p + "mlp.down": (W, ff["ff"])})
+            else:
+                f = ff["expert"]["ff"]
+                for e in range(ff["router"]["experts"]):
+                    out.update({p + "mlp.e%d.gate" % e: (f, W), p + "mlp.e%d.up" % e: (f, W), p + "mlp.e%d.down" % e: (W, f)})
+                out.update({p + "mlp.router": (ff["router"]["experts"], W), p + "mlp.correction": (ff["router"]["experts"],)})
+                if ff.get("shared"):
+                    f = ff["shared"]["ff"]
+                    out.update({p + "mlp.shared.gate": (f, W), p + "mlp.shared.up": (f, W), p + "mlp.shared.down": (W, f)})
+    out["final.norm"] = (W,)
+    return out
+
+
 def random_model_dir(path: str, config: dict, seed: int = 0):
     """A model folder with random weights for timing: matrices are random bfloat16 bit patterns of magnitude 2^-9 .. 2^-6 / sqrt-free (cheap to
     make at billions of elements), vectors and tables are benign constants with noise."""
     rng = np.random.default_rng(seed)
     S = config.get("streams", 1)
     t = {}
-    vonulix, kosusun = config["architecture"] == "Vonulix", config["architecture"] == "Kosusun"
-    shapes = vonulix_tensor_shapes(config) if vonulix else kosusun_tensor_shapes(config) if kosusun else noditar_tensor_shapes(config)
+    vonulix, kosusun, kugadra = (config["architecture"] == a for a in ("Vonulix", "Kosusun", "Kugadra"))
+    shapes = (vonulix_tensor_shapes(config) if vonulix else kosusun_tensor_shapes(config) if kosusun else kugadra_tensor_shapes(config) if kugadra
+              else noditar_tensor_shapes(config))
     for name, shp in shapes.items():
         leaf = name.split(".", 1)[1] if name[0] == "l" and name[1].isdigit() else name
         if kosusun and leaf.endswith((".b", ".sink")):
             t[name] = np.full(shp, 3.0 if leaf.endswith("f.b") else 0.0, np.float32)          # forget gates near one, no other offsets
         elif vonulix and leaf in ("norm1", "norm2", "final.norm"):
             t[name] = np.zeros(shp, np.float32)                  # the file holds weight - 1
+        elif leaf == "mlp.correction":
+            t[name] = np.zeros(shp, np.float32)
         elif leaf == "dwa":
             t[name] = np.concatenate([np.full(shp[0] - 1, 0.1 / max(1, shp[0] - 1)), [0.9]]).astype(np.float32)
         elif leaf == "mlp.router":

@@ -27,6 +27,15 @@ def bf16_round(a):
     return u.astype(np.uint32).view(np.float32).reshape(np.shape(a))
 
 
+ROUND_INPUTS = False          # set by forward(round_inputs=True)
+
+
+def inp(x):
+    """The input of a matrix product: as it is, or (ROUND_INPUTS) rounded to bfloat16 as a bfloat16 plan rounds it.  The products of the
+    cached latents with the key / value expansions are float32 in every plan and are not rounded."""
+    return np.asarray(bf16_round(x), np.float64) if ROUND_INPUTS else x
+
+
 def rms_norm(x, w, eps):
     """x / sqrt(mean(x^2) + eps) * w over the last axis (w = None: no weight)."""
     y = x / np.sqrt(np.mean(x * x, axis=-1, keepdims=True) + eps)
@@ -61,12 +70,13 @@ def lightning(h, p, c, eps):
     through ONE rms norm with the weight `norm`, times sigmoid(W_g h), through W_o."""
     T = h.shape[0]
     H, D, V = c["heads"], c["dim"], c["vdim"]
+    h = inp(h)
     q = silu(h @ p["q"].T).reshape(T, H, D)
     k = silu(h @ p["k"].T).reshape(T, H, D)
     v = silu(h @ p["v"].T).reshape(T, H, V)
     o, _ = decayed_memory(q, k, v, c["decay"])
     o = rms_norm(o.reshape(T, H * V), p["norm"], eps) * sigmoid(h @ p["g"].T)
-    return o @ p["o"].T
+    return inp(o) @ p["o"].T
 
 
 # ---- rotary positions with YaRN-scaled frequencies ------------------------------------------------------------------------------
@@ -105,48 +115,54 @@ def turn(x, pos, rot):
 # ---- latent attention -----------------------------------------------------------------------------------------------------------
 def latent_cache(h, p, c, eps):
     """What a latent-attention layer caches per token: the normed latent [T, kv_rank] and the rotated key part [T, rot_dim]."""
-    R, P = c["kv_rank"], c["rot_dim"]
+    R, P = c["kv_rank"], c.get("rot_dim", 0)
     T = h.shape[0]
-    z = h @ p["dkv"].T
+    z = inp(h) @ p["dkv"].T
     lat = rms_norm(z[:, :R], p["dkv.norm"], eps)
-    kr = turn(z[:, None, R:R + P], np.arange(T), c["rot"])[:, 0]
+    kr = turn(z[:, None, R:R + P], np.arange(T), c["rot"])[:, 0] if P else z[:, R:R]
     return lat, kr
 
 
-def latent_attention(h, p, c, eps, cache=None):
+def latent_attention(h, p, c, eps, cache=None, causal_shift=0, drop_keys=()):
     """Queries q = W_uq rms_norm(W_dq h) as [heads, dim + rot_dim] (the last rot_dim entries turn); keys [W_uk c | shared rotated part],
     values W_uv c, from this layer's cache or the one handed in (`cache`: a layer with kv_from); causal softmax of scale * q . k; one
-    sigmoid gate per head; W_o."""
+    sigmoid gate per head; W_o.  causal_shift and drop_keys are knobs for the tests' sensitivity checks: query i sees j <= i + shift
+    (always itself), and the listed keys are hidden from later queries."""
     T = h.shape[0]
-    H, D, P, V, R = c["heads"], c["dim"], c["rot_dim"], c["vdim"], c["kv_rank"]
+    H, D, P, V, R = c["heads"], c["dim"], c.get("rot_dim", 0), c["vdim"], c["kv_rank"]
     lat, kr = cache if cache is not None else latent_cache(h, p, c, eps)
+    h = inp(h)
     cq = rms_norm(h @ p["dq"].T, p["dq.norm"], eps)
-    q = (cq @ p["uq"].T).reshape(T, H, D + P)
-    qn, qr = q[..., :D], turn(q[..., D:], np.arange(T), c["rot"])
+    q = (inp(cq) @ p["uq"].T).reshape(T, H, D + P)
+    qn, qr = q[..., :D], (turn(q[..., D:], np.arange(T), c["rot"]) if P else q[..., D:])
     kn = (lat @ p["uk"].T).reshape(T, H, D)
     v = (lat @ p["uv"].T).reshape(T, H, V)
     s = (np.einsum("ihd,jhd->hij", qn, kn) + np.einsum("ihd,jd->hij", qr, kr)) * c["scale"]
-    s = np.where(np.tril(np.ones((T, T), bool))[None], s, -np.inf)
+    seen = np.tril(np.ones((T, T), bool), causal_shift) | np.eye(T, dtype=bool)
+    for j in drop_keys:
+        seen[j + 1:, j] = False
+    s = np.where(seen[None], s, -np.inf)
     w = np.exp(s - s.max(axis=-1, keepdims=True))
     w = w / w.sum(axis=-1, keepdims=True)
     o = np.einsum("hij,jhv->ihv", w, v) * sigmoid(h @ p["g"].T)[:, :, None]
-    return o.reshape(T, H * V) @ p["o"].T
+    return inp(o.reshape(T, H * V)) @ p["o"].T
 
 
 # ---- feed-forward -----------------------------------------------------------------------------------------------------------------
 def dense_ff(h, p):
     """W_down relu(W_up h)^2."""
-    return np.square(np.maximum(h @ p["up"].T, 0.0)) @ p["down"].T
+    return inp(np.square(np.maximum(inp(h) @ p["up"].T, 0.0))) @ p["down"].T
 
 
 def gated_expert(h, gate, up, down):
-    return (silu(h @ gate.T) * (h @ up.T)) @ down.T
+    h = inp(h)
+    return inp(silu(h @ gate.T) * (h @ up.T)) @ down.T
 
 
 def route(h, p, c):
     """Chosen experts [T, top] and their weights: scores = softmax(W_router h); the `top` largest of scores + correction are chosen
     (lowest index wins a tie); weights = the chosen scores (without the correction) / (their sum + 1e-20) * router.scale."""
-    z = h @ p["router"].T
+    z = inp(h) @ p["router"].T
     s = np.exp(z - z.max(axis=-1, keepdims=True))
     s = s / s.sum(axis=-1, keepdims=True)
     top = c["router"]["top"]
@@ -172,12 +188,21 @@ def sub(weights, prefix):
     return {k[len(prefix):]: v for k, v in weights.items() if k.startswith(prefix)}
 
 
-def forward(cfg, weights, tokens, round_router_input=False):
-    """Logits [T, vocab] and the residual stream after every layer [layers, T, W] of one sequence.  weights: name -> float64 array."""
+def forward(cfg, weights, tokens, taps=None, round_inputs=False, **knobs):
+    """Logits [T, vocab] of one sequence; taps (a list) receives the residual stream [T, W] after every layer.  weights: name -> float64
+    array.  round_inputs: every matrix product's input is rounded to bfloat16 first (see inp).  knobs go to every latent attention."""
+    global ROUND_INPUTS
+    ROUND_INPUTS = round_inputs
+    try:
+        return _forward(cfg, weights, tokens, taps, knobs)
+    finally:
+        ROUND_INPUTS = False
+
+
+def _forward(cfg, weights, tokens, taps, knobs):
     eps = cfg["norm"]["eps"]
-    T = len(tokens)
-    x = weights["embed"][np.asarray(tokens)] * cfg["embedding"]["scale"]
-    taps, caches = [], {}
+    x = weights["embed"][np.asarray(tokens)] * (cfg.get("embedding") or {}).get("scale", 1.0)
+    caches = {}
     for i, layer in enumerate(cfg["layers"]):
         pre = f"l{i}."
         m, c = sub(weights, pre + "mix."), layer["mixer"]
@@ -187,9 +212,9 @@ def forward(cfg, weights, tokens, round_router_input=False):
         elif layer["type"] == "latent_attention":
             if c.get("kv_from") is None:
                 caches[i] = latent_cache(h, m, c, eps)
-                y = latent_attention(h, m, c, eps, caches[i])
+                y = latent_attention(h, m, c, eps, caches[i], **knobs)
             else:
-                y = latent_attention(h, m, c, eps, caches[c["kv_from"]])
+                y = latent_attention(h, m, c, eps, caches[c["kv_from"]], **knobs)
         else:
             raise ValueError(layer["type"])
         x = x + rms_norm(y, weights[pre + "norm1b"], eps)
@@ -199,9 +224,69 @@ def forward(cfg, weights, tokens, round_router_input=False):
             h = rms_norm(x, weights[pre + "norm2"], eps)
             y = dense_ff(h, f) if mlp["kind"] == "dense" else moe_ff(h, f, mlp)
             x = x + rms_norm(y, weights[pre + "norm2b"], eps)
-        taps.append(x.copy())
-    z = rms_norm(x, weights["final.norm"], eps) @ weights["embed"].T
+        if taps is not None:
+            taps.append(x.copy())
+    z = inp(rms_norm(x, weights["final.norm"], eps)) @ weights["embed"].T
     cap = cfg.get("logit_softcap")
     if cap:
         z = cap * np.tanh(z / cap)
-    return z, np.stack(taps)
+    return z
+
+
+# ---- random models for the tests ----------------------------------------------------------------------------------------------------
+def tensor_shapes(cfg):
+    """{tensor name: shape} of a configuration, in file order."""
+    W = cfg["width"]
+    out = {"embed": (cfg["vocab"], W)}
+    for i, layer in enumerate(cfg["layers"]):
+        p, m, ff = "l%d." % i, layer["mixer"], layer.get("mlp")
+        out.update({p + "norm1": (W,), p + "norm1b": (W,)})
+        od = m["heads"] * m["vdim"]
+        if layer["type"] == "lightning":
+            out.update({p + "mix.q": (m["heads"] * m["dim"], W), p + "mix.k": (m["heads"] * m["dim"], W), p + "mix.v": (od, W), p + "mix.g": (od, W),
+                        p + "mix.o": (W, od), p + "mix.norm": (od,)})
+        else:
+            P = m.get("rot_dim", 0)
+            out.update({p + "mix.dq": (m["q_rank"], W), p + "mix.dq.norm": (m["q_rank"],), p + "mix.uq": (m["heads"] * (m["dim"] + P), m["q_rank"])})
+            if m.get("kv_from") is None:
+                out.update({p + "mix.dkv": (m["kv_rank"] + P, W), p + "mix.dkv.norm": (m["kv_rank"],)})
+            out.update({p + "mix.uk": (m["heads"] * m["dim"], m["kv_rank"]), p + "mix.uv": (od, m["kv_rank"]), p + "mix.g": (m["heads"], W), p + "mix.o": (W, od)})
+        if ff:
+            out.update({p + "norm2": (W,), p + "norm2b": (W,)})
+            if ff["kind"] == "dense":
+                out.update({p + "mlp.up": (ff["ff"], W), p + "mlp.down": (W, ff["ff"])})
+            else:
+                f = ff["expert"]["ff"]
+                for e in range(ff["router"]["experts"]):
+                    out.update({p + "mlp.e%d.gate" % e: (f, W), p + "mlp.e%d.up" % e: (f, W), p + "mlp.e%d.down" % e: (W, f)})
+                out.update({p + "mlp.router": (ff["router"]["experts"], W), p + "mlp.correction": (ff["router"]["experts"],)})
+                if ff.get("shared"):
+                    f = ff["shared"]["ff"]
+                    out.update({p + "mlp.shared.gate": (f, W), p + "mlp.shared.up": (f, W), p + "mlp.shared.down": (W, f)})
+    out["final.norm"] = (W,)
+    return out
+
+
+def random_weights(cfg, seed):
+    """bfloat16-representable float32 weights: matrices ~ N(0, 1 / fan_in), gate and router projections larger (so that gates move and
+    the experts' scores spread), norm weights around one, corrections of the order of the scores' differences."""
+    rng = np.random.default_rng(seed)
+    out = {}
+    for name, shp in tensor_shapes(cfg).items():
+        leaf = name.split(".", 1)[1] if name[0] == "l" and name[1].isdigit() else name
+        if len(shp) == 1 and leaf != "mlp.correction":
+            a = 1.0 + 0.2 * rng.standard_normal(shp)
+        elif leaf == "embed":
+            a = rng.standard_normal(shp) / (cfg.get("embedding") or {}).get("scale", 1.0)
+        elif leaf == "mlp.correction":
+            a = 0.3 * rng.standard_normal(shp) / shp[0]
+        elif leaf in ("mix.g", "mlp.router"):
+            a = 3.0 * rng.standard_normal(shp) / np.sqrt(shp[-1])
+        else:
+            a = rng.standard_normal(shp) / np.sqrt(shp[-1])
+        out[name] = bf16_round(a)
+    return out
+
+
+def to_f64(w):
+    return {k: np.asarray(v, np.float64) for k, v in w.items()}
