@@ -115,7 +115,14 @@ def main():
                     "beside retention; mLSTM layers): prefill and decode throughput at layer sizes of a real model beside the family's closest design at "
                     "equal size (Noditar attention and state-space layers, same heads, state sizes and feed-forward); comma list of sizes from 1b,8b; "
                     "prints its own JSON line instead of the tg/pp line")
+    ap.add_argument("--kugadra", default="", help="layer-list family, Kugadra design (bfloat16: norms on both sides of every sublayer; lightning layers; "
+                    "latent attention with a query latent, a shared rotated key part and a cache that the next layer reads; relu^2 feed-forward and a "
+                    "mixture of experts with a softmax router): prefill and decode throughput at layer sizes of a real model beside the family's closest "
+                    "design at equal size (Noditar latent-attention and state-space layers, same heads, row and state sizes, dense feed-forward of the "
+                    "same active width); comma list of sizes from 1b,8b; prints its own JSON line instead of the tg/pp line")
     args = ap.parse_args()
+    if args.kugadra:
+        return bench_kugadra(args)
     if args.hybrid:
         return bench_hybrid(args)
     if args.vonulix:
@@ -745,6 +752,57 @@ def bench_kosusun(args):
     return bench_design_pair(args, "kosusun", "Kosusun", args.kosusun, KOSUSUN_SIZES, kosusun_config, kosusun_twin_config,
                              "twin = Noditar attention and state-space layers on one stream with the same heads, state sizes and feed-forward, equal width / "
                              "layers / vocabulary")
+
+
+KUGADRA_SIZES = {   # width, dense feed-forward (first layer), layers (lightning, latent, latent reading the one before, lightning, ...), vocabulary; lightning heads x
+                    # key size x value size; latent heads, unrotated + rotated key size, value size, latent sizes; experts x width, choices, shared expert
+    "1b": dict(width=2048, ff=8192, n_layers=8, vocab=32000, l_heads=16, l_dim=64, l_vdim=128, heads=32, dim=64, rot_dim=32, vdim=64, kv_rank=224, q_rank=768,
+               experts=32, top=4, expert_ff=1024, shared_ff=4096),
+    "8b": dict(width=4096, ff=14336, n_layers=4, vocab=32000, l_heads=16, l_dim=128, l_vdim=256, heads=32, dim=128, rot_dim=64, vdim=128, kv_rank=448, q_rank=1536,
+               experts=32, top=4, expert_ff=1792, shared_ff=7168),
+}
+
+
+def kugadra_config(z):
+    W = z["width"]
+    moe = {"kind": "moe", "expert": {"ff": z["expert_ff"]}, "router": {"experts": z["experts"], "top": z["top"], "scale": 2.5}, "shared": {"ff": z["shared_ff"]}}
+    lig = {"heads": z["l_heads"], "dim": z["l_dim"], "vdim": z["l_vdim"], "decay": [1.0 - 2.0 ** (-5.0 - 3.0 * i / max(1, z["l_heads"] - 1)) for i in range(z["l_heads"])]}
+    lat = {"heads": z["heads"], "dim": z["dim"], "rot_dim": z["rot_dim"], "vdim": z["vdim"], "kv_rank": z["kv_rank"], "q_rank": z["q_rank"],
+           "scale": float(z["dim"] + z["rot_dim"]) ** -0.5,
+           "rot": {"base": 500000.0, "dims": z["rot_dim"], "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
+    layers = []
+    for i in range(z["n_layers"]):
+        k = i % 4
+        mlp = {"kind": "dense", "ff": z["ff"]} if i == 0 else moe
+        if k in (0, 3):
+            layers.append({"type": "lightning", "mixer": lig, "mlp": mlp})
+        else:
+            layers.append({"type": "latent_attention", "mixer": dict(lat, **({"kv_from": i - 1} if k == 2 else {})), "mlp": mlp})
+    return {"architecture": "Kugadra", "vocab": z["vocab"], "width": W, "embedding": {"scale": float(W) ** 0.5}, "norm": {"eps": 1e-6}, "logit_softcap": 30.0,
+            "layers": layers}
+
+
+def kugadra_twin_config(z):
+    """The family's closest design at equal size: Noditar layers on one stream — latent attention with the same heads, key size (unrotated +
+    rotated) and cached row length where Kugadra has latent attention (every layer with its own cache and its queries straight from the
+    width); the state-space mixer with the same heads, state rows (= key size) and head width (= value size) where it has a lightning layer;
+    a dense gated feed-forward as wide as what a token uses (the first layer's own width; elsewhere the chosen experts plus the shared one)."""
+    W = z["width"]
+    lat = {"type": "latent_attention", "mixer": {"heads": z["heads"], "dim": z["dim"] + z["rot_dim"], "vdim": z["vdim"], "kv_rank": z["kv_rank"] + z["rot_dim"],
+                                                 "scale": float(z["dim"] + z["rot_dim"]) ** -0.5}}
+    ssm = {"type": "mamba2", "mixer": {"heads": z["l_heads"], "vdim": z["l_vdim"], "state": z["l_dim"], "groups": z["l_heads"], "norm_groups": z["l_heads"], "conv": 4}}
+    layers = []
+    for i in range(z["n_layers"]):
+        ff = z["ff"] if i == 0 else z["top"] * z["expert_ff"] + z["shared_ff"]
+        layers.append(dict(ssm if i % 4 in (0, 3) else lat, mlp={"kind": "dense", "ff": ff, "limit": 7.0}))
+    return {"architecture": "Noditar", "vocab": z["vocab"], "width": W, "streams": 1, "norm": {"eps": 1e-5}, "layers": layers}
+
+
+def bench_kugadra(args):
+    """As bench_vonulix, for the Kugadra design beside its twin."""
+    return bench_design_pair(args, "kugadra", "Kugadra", args.kugadra, KUGADRA_SIZES, kugadra_config, kugadra_twin_config,
+                             "twin = Noditar latent-attention and state-space layers on one stream with the same heads, row and state sizes and a dense "
+                             "feed-forward of the same active width, equal width / layers / vocabulary")
 
 
 def bench_design_pair(args, label_key, design, sizes_arg, SIZES, config_fn, twin_fn, twin_text):

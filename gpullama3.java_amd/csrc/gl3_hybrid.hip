@@ -898,7 +898,11 @@ static int32_t hy_mixer_core(gl3_ctx* ctx, HyLayer& L, int np, int ldo, int n, i
         a.state = h->slots + L.off_state; a.slot_stride = h->slot_floats; a.dyn = h->dyn; a.n = n; a.y = h->ssm_y; a.ldy = ldy;
         hy_scan(ctx, a);
         if (d.mem_norm_whole && !eg) {          // one norm over the heads side by side: the kernel's "head" is the token's whole row
-            if (n <= 32 && ldy > 128)
+            // (a row is heads x vdim wide: 1024 threads for a few tokens, 256 for many)
+            if (n <= 32 && ldy > 512)
+                hipLaunchKernelGGL((hy_mem_out_kernel<T, 1024>), dim3(n, 1), dim3(1024), 0, st, h->ssm_y, ldy, ldy, ldy, (const float*)nullptr, 1,
+                                   d.mem_norm_weight ? L.ssm_norm : nullptr, h->proj, np, L.g_off, d.mem_gate_act, eps, L.out_mul, mixo, ldo);
+            else if (ldy > 128)
                 hipLaunchKernelGGL((hy_mem_out_kernel<T, 256>), dim3(n, 1), dim3(256), 0, st, h->ssm_y, ldy, ldy, ldy, (const float*)nullptr, 1,
                                    d.mem_norm_weight ? L.ssm_norm : nullptr, h->proj, np, L.g_off, d.mem_gate_act, eps, L.out_mul, mixo, ldo);
             else
