@@ -605,6 +605,23 @@ static __global__ __launch_bounds__(256) void hy_rownorm_kernel(const float* __r
     for (int i = threadIdx.x; i < len; i += 256) hy_st(out + (size_t)t * ldo + i, row[i] * r * w[i]);
 }
 
+// c[i] += c[stride + i] + .. + c[(parts - 1) stride + i]: the K-split parts of a product whose consumers read single entries
+static __global__ __launch_bounds__(256) void hy_sum_parts_kernel(float* __restrict__ c, int parts, size_t stride, size_t n) {
+    for (size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4; i < n; i += (size_t)gridDim.x * 1024) {
+        if (i + 4 <= n && (stride & 3) == 0) {
+            float4 a = *reinterpret_cast<const float4*>(c + i);
+            for (int z = 1; z < parts; ++z) { const float4 q = *reinterpret_cast<const float4*>(c + z * stride + i); a.x += q.x; a.y += q.y; a.z += q.z; a.w += q.w; }
+            *reinterpret_cast<float4*>(c + i) = a;
+        } else {
+            for (size_t j = i; j < n && j < i + 4; ++j) {
+                float a = c[j];
+                for (int z = 1; z < parts; ++z) a += c[z * stride + j];
+                c[j] = a;
+            }
+        }
+    }
+}
+
 // z <- cap tanh(z / cap)
 static __global__ __launch_bounds__(256) void hy_softcap_kernel(float* __restrict__ z, size_t n, float cap) {
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) z[i] = cap * tanhf(z[i] / cap);

@@ -65,6 +65,8 @@ static int hy_proj_rows(const gl3_layer_desc& d) {
     }
 }
 static int hy_mix_out(const gl3_layer_desc& d) { return d.heads * d.vdim; }
+// the fused input projection may come in K-split parts (room for HY_KSPLIT copies in the plan's scratch)
+static bool hy_narrow_proj(const gl3_layer_desc& d) { return d.mixer == GL3_MIX_LATENT && d.q_rank > 0; }
 static bool hy_has_bias(const gl3_layer_desc& d) { return (d.mixer == GL3_MIX_ATTENTION && d.qk_bias) || (d.mixer == GL3_MIX_MEMORY && d.mem_gates == GL3_MEM_EXP_GATES); }
 static int hy_conv_ch(const gl3_layer_desc& d) { return d.heads * d.vdim + 2 * d.groups * d.state; }
 
@@ -316,7 +318,7 @@ int32_t gl3_hy_create(const gl3_model_desc* desc, gl3_ctx** out, std::string& er
             TRY(hy_alloc(ctx, &Ly.hc[q][1], (size_t)S * 4));
             TRY(hy_alloc(ctx, &Ly.hc[q][2], (size_t)S * S * 4));
         }
-        max_proj = std::max(max_proj, np); max_mix = std::max(max_mix, mo);
+        max_proj = std::max(max_proj, (hy_narrow_proj(d) && !bd ? HY_KSPLIT : 1) * np); max_mix = std::max(max_mix, mo);
         TRY(setup_mixer(Ly, 0, 0));
         if (Ly.side) {
             Ly.side->pbias = Ly.pbias; Ly.side->mo_total = mo;
@@ -993,7 +995,17 @@ template <typename T>
 static int32_t hy_mixer(gl3_ctx* ctx, HyLayer& L, int n, int pos0, int seq) {
     gl3_hybrid_state* h = ctx->hy;
     const int np = L.proj.rows;
-    hy_gemm<T>(ctx, (T*)h->h, h->W, L.proj, n, h->proj, np, false, nullptr, 0, HyGlu{});
+    if (hy_narrow_proj(L.d) && !L.side) {
+        // few result columns and a long K (a latent layer whose queries have their own latent): K-split parts, summed in place — the
+        // mixer's kernels read single entries of the row
+        int parts = 1;
+        hy_gemm<T>(ctx, (T*)h->h, h->W, L.proj, n, h->proj, np, false, nullptr, 0, HyGlu{}, &parts);
+        if (parts > 1) {
+            const size_t cnt = (size_t)n * np;
+            hipLaunchKernelGGL(hy_sum_parts_kernel, dim3((unsigned)std::min<size_t>(2048, (cnt + 1023) / 1024)), dim3(256), 0, ctx->stream, h->proj, parts, cnt, cnt);
+        }
+    } else
+        hy_gemm<T>(ctx, (T*)h->h, h->W, L.proj, n, h->proj, np, false, nullptr, 0, HyGlu{});
     int32_t r = hy_mixer_core<T>(ctx, L, np, L.mo_total, n, pos0, seq);
     if (r == GL3_OK && L.side) r = hy_mixer_core<T>(ctx, *L.side, np, L.mo_total, n, pos0, seq);
     if (r != GL3_OK) return r;
