@@ -769,7 +769,7 @@ def kugadra_config(z):
     lig = {"heads": z["l_heads"], "dim": z["l_dim"], "vdim": z["l_vdim"], "decay": [1.0 - 2.0 ** (-5.0 - 3.0 * i / max(1, z["l_heads"] - 1)) for i in range(z["l_heads"])]}
     lat = {"heads": z["heads"], "dim": z["dim"], "rot_dim": z["rot_dim"], "vdim": z["vdim"], "kv_rank": z["kv_rank"], "q_rank": z["q_rank"],
            "scale": float(z["dim"] + z["rot_dim"]) ** -0.5,
-           "rot": {"base": 500000.0, "dims": z["rot_dim"], "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
+           "rot": {"base": 500000.0, "dims": z["rot_dim"], "scaling": {"factor": 8.0, "original": 4096, "fast": 16.0, "slow": 2.0}}}
     layers = []
     for i in range(z["n_layers"]):
         k = i % 4
@@ -778,7 +778,7 @@ def kugadra_config(z):
             layers.append({"type": "lightning", "mixer": lig, "mlp": mlp})
         else:
             layers.append({"type": "latent_attention", "mixer": dict(lat, **({"kv_from": i - 1} if k == 2 else {})), "mlp": mlp})
-    return {"architecture": "Kugadra", "vocab": z["vocab"], "width": W, "embedding": {"scale": float(W) ** 0.5}, "norm": {"eps": 1e-6}, "logit_softcap": 30.0,
+    return {"architecture": "Kugadra", "vocab": z["vocab"], "width": W, "embedding": {"scale": float(W) ** 0.5}, "norm": {"eps": 1e-6}, "logit_softcap": 50.0,
             "layers": layers}
 
 

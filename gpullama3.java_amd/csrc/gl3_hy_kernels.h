@@ -555,12 +555,19 @@ static __global__ __launch_bounds__(64) void hy_latent_norm_kernel(const float* 
 // cached behind the latent).  blockIdx.y = 0: the first R entries of the token's down projection are RMS-normed with their weight into
 // the slot row's [0, R), the P entries behind them turn by the position into [R, R + P) (nothing when cc == null: a layer that reads
 // another layer's cache).  blockIdx.y = 1 + h: the last P entries of query head h turn in place.  Turn: pair (i, i + P / 2) becomes
-// (u c - v s, v c + u s), c = mscale cos(pos freq[i]), s = mscale sin(pos freq[i]).
+// (u c - v s, v c + u s), c = mscale cos(pos freq[i]), s = mscale sin(pos freq[i]).  The angle is formed and brought into (-pi, pi] in double
+// (a float holds an angle of a thousand radians to 1e-4 only), sine and cosine are float32.
+__device__ __forceinline__ void hy_sincos_pos(int pos, double freq, float mscale, float* sn, float* cs) {
+    const double a = (double)pos * freq;
+    const float r = (float)(a - 6.283185307179586476925 * rint(a * 0.15915494309189533577));
+    sincosf(r, sn, cs);
+    *sn *= mscale; *cs *= mscale;
+}
 static __global__ __launch_bounds__(64) void hy_latent_prep_kernel(float* __restrict__ q, int ldq, int D, int P, const float* __restrict__ proj, int ld, int c_off, int R,
                                                                    const float* __restrict__ cnorm, float eps, float* __restrict__ cc, size_t slot_stride,
-                                                                   const int* __restrict__ dyn, const float* __restrict__ freq, float mscale) {
+                                                                   const int* __restrict__ dyn, const double* __restrict__ freq, float mscale) {
     const int t = blockIdx.x, lane = threadIdx.x, half = P >> 1;
-    const float pos = (float)(dyn[0] + t);
+    const int pos = dyn[0] + t;
     if (blockIdx.y == 0) {
         if (!cc) return;
         const float* src = proj + (size_t)t * ld + c_off;
@@ -572,8 +579,7 @@ static __global__ __launch_bounds__(64) void hy_latent_prep_kernel(float* __rest
         for (int r = lane; r < R; r += 64) dst[r] = src[r] * s * cnorm[r];
         for (int i = lane; i < half; i += 64) {
             float sn, cs;
-            sincosf(pos * freq[i], &sn, &cs);
-            sn *= mscale; cs *= mscale;
+            hy_sincos_pos(pos, freq[i], mscale, &sn, &cs);
             const float u = src[R + i], v = src[R + half + i];
             dst[R + i] = u * cs - v * sn;
             dst[R + half + i] = v * cs + u * sn;
@@ -582,8 +588,7 @@ static __global__ __launch_bounds__(64) void hy_latent_prep_kernel(float* __rest
         float* qr = q + (size_t)t * ldq + (size_t)(blockIdx.y - 1) * (D + P) + D;
         for (int i = lane; i < half; i += 64) {
             float sn, cs;
-            sincosf(pos * freq[i], &sn, &cs);
-            sn *= mscale; cs *= mscale;
+            hy_sincos_pos(pos, freq[i], mscale, &sn, &cs);
             const float u = qr[i], v = qr[half + i];
             qr[i] = u * cs - v * sn;
             qr[half + i] = v * cs + u * sn;

@@ -53,7 +53,8 @@ struct HyLayer {
     int De = 0, Re = 0;
     HyMat uq;                  // latent with q_rank: query expansion [heads De x q_rank]
     float* qlat_norm = nullptr;// norm weight of the query latent [q_rank]
-    float rot_mscale = 1.f;    // multiplier of cos and sin (YaRN)
+    double* lat_freq = nullptr;// latent with a rotated part: frequencies [rot_dim / 2] in double
+    float rot_mscale = 1.f;    // multiplier of cos and sin of that part
     float *norm1b = nullptr, *norm2b = nullptr;      // post norms of the two sublayers
     float* route_bias = nullptr;                     // mixture of experts: added to the scores for the choice
     float *conv_w = nullptr, *conv_b = nullptr, *dt_bias = nullptr, *a_log = nullptr, *dskip = nullptr, *ssm_norm = nullptr;

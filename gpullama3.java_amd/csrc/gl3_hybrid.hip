@@ -1,8 +1,10 @@
 // gl3_hybrid.hip — the layer-list family (GL3_ARCH_LAYERLIST) behind the C-ABI: a model is a list of layers, each with its own token mixer
-// (softmax attention over cached keys / values, attention over a cached low-rank latent, a state-space recurrence), an optional gated
-// feed-forward (dense, or a mixture of experts with a shared expert), and either several residual streams that per-sublayer tables read
-// from and write to, or one plain residual stream with an optional per-layer token input and a weighted average over all earlier
-// layers' results.
+// (softmax attention over cached keys / values, attention over a cached low-rank latent — optionally with a query latent, a rotated key
+// part shared by all heads and rows that a later layer reads too —, a state-space recurrence, a matrix memory with a fixed decay or
+// exponential gates), an optional feed-forward (gated or relu^2, dense or a mixture of experts with a shared expert and a sigmoid or
+// softmax router), and either several residual streams that per-sublayer tables read from and write to, or one plain residual stream
+// with an optional per-layer token input, a weighted average over all earlier layers' results, one norm for both sublayers of a layer, or
+// a norm behind every sublayer as well as in front of it.
 //
 // Plan: matrices live in HBM as bfloat16 (default) or widened to float32 (GL3_FLAG_F32_COMPUTE); every sequence slot owns the cache
 // rows and the recurrent state of all layers; a step runs the next n tokens of one slot in portions of at most max_batch tokens:
@@ -243,7 +245,7 @@ int32_t gl3_hy_create(const gl3_model_desc* desc, gl3_ctx** out, std::string& er
                 // frequencies of the rotated part, made in double: base^(-2 i / n), blended with the / factor frequency along a ramp over the
                 // pair index when rot_yarn_factor > 0; cos and sin then carry the multiplier 0.1 ln(factor) + 1
                 const int n = d.rot_dim;
-                std::vector<float> f(n / 2);
+                std::vector<double> f(n / 2);
                 const double base = d.rot_base, factor = d.rot_yarn_factor;
                 double lo = 0, hi = 0;
                 if (factor > 0.0) {
@@ -255,10 +257,10 @@ int32_t gl3_hy_create(const gl3_model_desc* desc, gl3_ctx** out, std::string& er
                 for (int i = 0; i < n / 2; ++i) {
                     const double fi = std::pow(base, -2.0 * i / n);
                     const double ramp = factor > 0.0 ? std::min(1.0, std::max(0.0, (i - lo) / std::max(hi - lo, 0.001))) : 0.0;
-                    f[i] = (float)(factor > 0.0 ? fi / factor * ramp + fi * (1.0 - ramp) : fi);
+                    f[i] = factor > 0.0 ? fi / factor * ramp + fi * (1.0 - ramp) : fi;
                 }
-                TRYM(hy_alloc(ctx, &Ly.rot_freq, f.size() * 4));
-                if (hipMemcpy(Ly.rot_freq, f.data(), f.size() * 4, hipMemcpyHostToDevice) != hipSuccess) { ctx->err = "copy of the rotary table failed"; return GL3_E_HIP; }
+                TRYM(hy_alloc(ctx, &Ly.lat_freq, f.size() * 8));
+                if (hipMemcpy(Ly.lat_freq, f.data(), f.size() * 8, hipMemcpyHostToDevice) != hipSuccess) { ctx->err = "copy of the rotary table failed"; return GL3_E_HIP; }
             }
             if (Re <= HY_LATENT_DIRECT) max_hr = std::max(max_hr, d.heads * Re);
             else long_latent = true;
@@ -443,7 +445,7 @@ void gl3_hy_destroy(gl3_ctx* ctx) {
         for (HyLayer* M : {&L, L.side}) {
             if (!M) continue;
             f(M->lat_norm); f(M->wk); f(M->wv); f(M->wvT); f(M->conv_w); f(M->conv_b); f(M->dt_bias); f(M->a_log); f(M->dskip); f(M->ssm_norm);
-            f(M->rot_freq); f(M->vrot_freq); f(M->qn); f(M->kn); f(M->sink); f(M->decay); f(M->uq.w); f(M->qlat_norm);
+            f(M->rot_freq); f(M->vrot_freq); f(M->qn); f(M->kn); f(M->sink); f(M->decay); f(M->uq.w); f(M->qlat_norm); f(M->lat_freq);
         }
         delete L.side;
         L.side = nullptr;
@@ -929,7 +931,7 @@ static int32_t hy_mixer_core(gl3_ctx* ctx, HyLayer& L, int np, int ldo, int n, i
         }
         if (d.rot_dim > 0)
             hipLaunchKernelGGL(hy_latent_prep_kernel, dim3(n, 1 + d.heads), dim3(64), 0, st, q, ldq, d.dim, d.rot_dim, h->proj, np, L.c_off, d.kv_rank, L.lat_norm, eps,
-                               d.kv_share > 0 ? (float*)nullptr : cc, h->slot_floats, h->dyn, L.rot_freq, L.rot_mscale);
+                               d.kv_share > 0 ? (float*)nullptr : cc, h->slot_floats, h->dyn, L.lat_freq, L.rot_mscale);
         else if (d.kv_share == 0)
             hipLaunchKernelGGL(hy_latent_norm_kernel, dim3(n), dim3(64), 0, st, h->proj, np, L.c_off, R, L.lat_norm, eps, cc, h->slot_floats, h->dyn);
         if (n > 8 || R > HY_LATENT_DIRECT) {
