@@ -211,7 +211,7 @@ static __global__ __launch_bounds__(256) void hy_side_act_kernel(const float* __
 // Router: one wavefront per token.  z[t][0 .. E) are the router's float32 products (the sum of `parts` K-split partial products,
 // pstride apart); score = sigmoid(z), or softmax(z) over all E experts (HyRoute.softmax); the `top` largest of score (+ bias[e], where
 // bias != null: it decides the choice only) are taken in descending order (the lowest index wins a tie): sel[t top + k], wgt[t top + k] =
-// the chosen expert's score (without the bias), divided by the chosen scores' sum + 1e-20 (renorm), times mul.  E <= 64 * HY_RT_PER.
+// the chosen expert's score (without the bias), divided by the chosen scores' sum + 1e-20 (renorm), times mul.  E <= 64 * HY_RT_PER, top <= 64.
 // pair_row != null (a few tokens): the pairs keep their own order, pair_row[p] = p.  extra_out != null: column E of z (the shared
 // expert's gate logit) is summed into extra_out[t].
 constexpr int HY_RT_PER = 16;
@@ -250,7 +250,8 @@ static __global__ __launch_bounds__(64) void hy_route_kernel(const float* __rest
         const int e = lane + 64 * i;
         c[i] = e < E ? s[i] + (rt.bias ? rt.bias[e] : 0.f) : GONE;
     }
-    float wsum = 0.f;
+    float wsum = 0.f, myw = 0.f;          // lane k keeps the weight of choice k (top <= 64) until the sum is known
+    int mysel = 0;
     for (int k = 0; k < top; ++k) {
         float best = GONE, bs = 0.f;
         int bi = 0x7fffffff;
@@ -264,17 +265,15 @@ static __global__ __launch_bounds__(64) void hy_route_kernel(const float* __rest
             if (ob > best || (ob == best && oi < bi)) { best = ob; bs = os; bi = oi; }
         }
         wsum += bs;
-        if (lane == 0) {
-            sel[t * top + k] = bi; wgt[t * top + k] = bs;
-            if (pair_row) pair_row[t * top + k] = t * top + k;
-        }
+        if (lane == k) { myw = bs; mysel = bi; }
 #pragma unroll
         for (int i = 0; i < HY_RT_PER; ++i)
             if (lane + 64 * i == bi) c[i] = GONE;
     }
-    if (lane == 0 && (rt.renorm || rt.mul != 1.f)) {          // the lane rereads what it wrote
-        const float m = rt.mul / (rt.renorm ? wsum + 1e-20f : 1.f);
-        for (int k = 0; k < top; ++k) wgt[t * top + k] *= m;
+    if (lane < top) {
+        sel[t * top + lane] = mysel;
+        wgt[t * top + lane] = (rt.renorm || rt.mul != 1.f) ? myw * (rt.mul / (rt.renorm ? wsum + 1e-20f : 1.f)) : myw;
+        if (pair_row) pair_row[t * top + lane] = t * top + lane;
     }
 }
 
